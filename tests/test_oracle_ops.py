@@ -1,0 +1,261 @@
+"""Pins each oracle function against something independent of its own formula:
+library routines, float64 brute force, closed forms and special cases."""
+import numpy as np
+import pytest
+import torch
+
+import pyoracle as po
+from synth import quantize_u8
+
+rng = np.random.default_rng(7)
+
+
+def h(x):
+    return np.asarray(x, np.float32).astype(np.float16)
+
+
+# ---------------------------------------------------------------- layernorm
+def test_layernorm_f32_matches_torch():
+    x = rng.standard_normal((5, 768)).astype(np.float32) * 3 + 1
+    g = rng.standard_normal(768).astype(np.float32)
+    b = rng.standard_normal(768).astype(np.float32)
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x), (768,), torch.from_numpy(g),
+                                         torch.from_numpy(b), 1e-5).numpy()
+    assert np.allclose(po.layernorm_f32(x, g, b), ref, atol=2e-6, rtol=1e-5)
+
+
+def test_layernorm_f16_rounding_points():
+    """normalise in fp32 -> half -> *gamma in half -> +beta in half
+    (kernels/cuda/layer_norm.cu:60-69)."""
+    x = h(rng.standard_normal((3, 2048)) * 2)
+    g = h(1 + 0.1 * rng.standard_normal(2048))
+    b = h(0.1 * rng.standard_normal(2048))
+    xf = x.astype(np.float64)
+    mean = xf.mean(axis=1, keepdims=True)
+    var = xf.var(axis=1, keepdims=True)
+    n = ((xf - mean) / np.sqrt(var + 1e-5)).astype(np.float32).astype(np.float16)
+    ref = ((n * g).astype(np.float16) + b).astype(np.float16)
+    got = po.layernorm_f16(x, g, b)
+    # the fp32 normalised value can sit next to a half rounding boundary: allow 1 ulp on a few
+    diff = np.abs(got.view(np.int16).astype(np.int32) - ref.view(np.int16).astype(np.int32))
+    assert diff.max() <= 1 and (diff > 0).mean() < 0.01
+
+
+def test_layernorm_special_cases():
+    C = 512
+    g = h(rng.standard_normal(C))
+    b = h(rng.standard_normal(C))
+    const = np.full(C, 3.25, np.float16)
+    assert np.array_equal(po.layernorm_f16(const, g, b), b)  # zero variance -> beta
+    x = h(rng.standard_normal(C))
+    y = po.layernorm_f16(x, np.ones(C, np.float16), np.zeros(C, np.float16)).astype(np.float64)
+    assert abs(y.mean()) < 2e-3 and abs(y.var() - 1) < 5e-3
+
+
+def test_groupnorm_matches_torch():
+    H, S, T = 40, 64, 3
+    x = rng.standard_normal((T, H * S)).astype(np.float32) * 2
+    g = rng.standard_normal(H * S).astype(np.float32)
+    b = rng.standard_normal(H * S).astype(np.float32)
+    ref = torch.nn.functional.group_norm(torch.from_numpy(x), H, torch.from_numpy(g),
+                                         torch.from_numpy(b), 1e-5).numpy()
+    assert np.allclose(po.groupnorm_f32(x, H, g, b), ref, atol=3e-6, rtol=1e-5)
+
+
+# ---------------------------------------------------------------------- mix
+def test_mix_closed_form_and_limits():
+    C = 1024
+    xx, sx = h(rng.standard_normal(C)), h(rng.standard_normal(C))
+    assert np.array_equal(po.mix_f16(xx, sx, np.ones(C, np.float16)), xx)   # m=1 -> xx
+    assert np.array_equal(po.mix_f16(xx, sx, np.zeros(C, np.float16)), sx)  # m=0 -> sx
+    m = h(rng.uniform(0, 1, C))
+    ref = ((xx * m).astype(np.float16) + (sx * (np.float16(1) - m).astype(np.float16)).astype(np.float16))
+    assert np.array_equal(po.mix_f16(xx, sx, m), ref.astype(np.float16))
+    # broadcast of the mix vector over rows (att_seq.cu:34-36: mix[i % C])
+    X, Sx = h(rng.standard_normal((4, C))), h(rng.standard_normal((4, C)))
+    got = po.mix_f16(X, Sx, m)
+    for t in range(4):
+        assert np.array_equal(got[t], po.mix_f16(X[t], Sx[t], m))
+
+
+# --------------------------------------------------------------------- gemm
+@pytest.mark.parametrize("T,K,N", [(1, 2048, 512), (3, 300, 70), (9, 64, 257)])
+def test_gemm_f16_against_float64(T, K, N):
+    x = h(rng.standard_normal((T, K)))
+    W = h(rng.standard_normal((K, N)) * 0.02)
+    ref = x.astype(np.float64) @ W.astype(np.float64)
+    got = po.gemm_f16(x, W, "f32")
+    assert np.allclose(got, ref, atol=1e-5 * np.sqrt(K), rtol=1e-5)
+    got16 = po.gemm_f16(x, W, "f16")
+    assert np.array_equal(got16, got.astype(np.float16))  # one rounding of the fp32 sum
+    if T == 1:
+        assert np.array_equal(po.gemm_f16(x[0], W, "f32"), got[0])
+    # a transposed-operand mistake would fail this asymmetric case
+    e = np.zeros((1, K), np.float16)
+    e[0, 5] = 1
+    assert np.array_equal(po.gemm_f16(e, W, "f16")[0], W[5])
+
+
+def test_gemm_f32_against_float64():
+    x = rng.standard_normal((2, 333)).astype(np.float32)
+    W = rng.standard_normal((333, 129)).astype(np.float32)
+    assert np.allclose(po.gemm_f32(x, W), x.astype(np.float64) @ W.astype(np.float64), atol=1e-4)
+
+
+# -------------------------------------------------------------- elementwise
+def test_sigmoid_relu2_silu_closed_forms():
+    x = h(np.linspace(-12, 12, 4001))
+    xd = x.astype(np.float64)
+    s = po.sigmoid_f16(x)
+    ref = (1 / (1 + np.exp(-xd))).astype(np.float32).astype(np.float16)
+    assert np.array_equal(s, ref)
+    assert po.sigmoid_f16(h([0.0]))[0] == np.float16(0.5)
+    r2 = po.relu_square_f16(x)
+    assert np.array_equal(r2, np.where(xd > 0, (x * x).astype(np.float16), np.float16(0)))
+    assert np.isinf(po.relu_square_f16(h([256.0]))[0])  # overflow above |x|>255.9 (ffn.cu:42-49)
+    si = po.silu_f16(x)
+    e = np.exp(-x.astype(np.float32)).astype(np.float16)
+    ref = (x.astype(np.float32) / (np.float16(1) + e).astype(np.float16).astype(np.float32)).astype(np.float16)
+    dif = np.abs(si.view(np.int16).astype(int) - ref.view(np.int16).astype(int))
+    assert dif.max() <= 1  # expf vs numpy exp may differ in the last fp32 bit
+    assert np.allclose(si.astype(np.float64), xd / (1 + np.exp(-xd)), rtol=3e-3, atol=1e-3)
+
+
+def test_known_answer_one_half():
+    """tests/test_ops.cpp:9-16: fill_(1); scalar_div_(2) == 0.5 in fp16."""
+    one, two = 0x3C00, 0x4000
+    assert po.lib.orc_hdiv(one, two) == np.float16(0.5).view(np.uint16)
+
+
+# ---------------------------------------------------------------------- WKV
+def _wkv4_closed_form(k, v, w, u):
+    """wkv_t = (sum_{i<t} e^{(t-1-i)w + k_i} v_i + e^{u+k_t} v_t) / (same without v), float64."""
+    T, C = k.shape
+    out = np.zeros((T, C))
+    for t in range(T):
+        num = np.exp(u + k[t]) * v[t]
+        den = np.exp(u + k[t])
+        for i in range(t):
+            e = np.exp((t - 1 - i) * w + k[i])
+            num += e * v[i]
+            den += e
+        out[t] = num / den
+    return out
+
+
+def test_wkv4_recurrence_matches_closed_form_and_first_step_is_v():
+    T, C = 12, 64
+    k = rng.standard_normal((T, C)).astype(np.float32)
+    v = rng.standard_normal((T, C)).astype(np.float32)
+    w = (-np.exp(rng.uniform(-5, 1, C))).astype(np.float32)
+    u = rng.uniform(-1, 1, C).astype(np.float32)
+    ref = _wkv4_closed_form(k.astype(np.float64), v.astype(np.float64), w.astype(np.float64),
+                            u.astype(np.float64))
+    aa, bb = np.zeros(C, np.float32), np.zeros(C, np.float32)
+    pp = np.full(C, -1e30, np.float32)
+    for t in range(T):
+        r, aa, bb, pp = po.wkv4_one_f16(u, w, k[t], v[t], aa, bb, pp, np.ones(C, np.float16))
+        # r = h(1 * h(wkv)) = h(wkv)
+        assert np.allclose(r.astype(np.float64), ref[t], rtol=2e-3, atol=2e-3), t
+        if t == 0:
+            assert np.array_equal(r, v[0].astype(np.float16))  # empty state: wkv_0 = v_0
+    # the state after T steps, in shift-free form, equals the direct sums
+    num = sum(np.exp((T - 1 - i) * w.astype(np.float64) + k[i]) * v[i] for i in range(T))
+    den = sum(np.exp((T - 1 - i) * w.astype(np.float64) + k[i]) for i in range(T))
+    assert np.allclose(aa * np.exp(pp.astype(np.float64)), num, rtol=1e-4)
+    assert np.allclose(bb * np.exp(pp.astype(np.float64)), den, rtol=1e-4)
+
+
+def test_wkv4_independent_of_max_shift():
+    C = 32
+    k, v = rng.standard_normal(C).astype(np.float32), rng.standard_normal(C).astype(np.float32)
+    w = (-np.exp(rng.uniform(-5, 1, C))).astype(np.float32)
+    u = rng.uniform(-1, 1, C).astype(np.float32)
+    aa, bb = rng.uniform(0.5, 2, C).astype(np.float32), rng.uniform(0.5, 2, C).astype(np.float32)
+    pp = rng.standard_normal(C).astype(np.float32)
+    one = np.ones(C, np.float16)
+    r1, a1, b1, p1 = po.wkv4_one_f16(u, w, k, v, aa, bb, pp, one)
+    d = np.float32(1.5)  # the same state written with another exponent offset
+    r2, a2, b2, p2 = po.wkv4_one_f16(u, w, k, v, aa * np.exp(d), bb * np.exp(d), pp - d, one)
+    assert np.abs(r1.astype(np.float32) - r2.astype(np.float32)).max() <= 2e-3
+    assert np.allclose(a1 * np.exp(p1.astype(np.float64)), a2 * np.exp(p2.astype(np.float64)), rtol=1e-4)
+
+
+def _wkv5_brute(r, k, v, w, u, s0):
+    """y_t = r_t . (diag(u) k_t v_t^T + S_{t-1});  S_t = diag(w) S_{t-1} + k_t v_t^T, float64,
+    S indexed [head][key][value]."""
+    T, C = r.shape
+    H, S = w.shape
+    s = s0.astype(np.float64).copy()
+    y = np.zeros((T, C))
+    for t in range(T):
+        for hd in range(H):
+            sl = slice(hd * S, (hd + 1) * S)
+            a = np.outer(k[t, sl], v[t, sl])
+            y[t, sl] = r[t, sl] @ (u[hd][:, None] * a + s[hd])
+            s[hd] = w[hd][:, None] * s[hd] + a
+    return y, s
+
+
+def test_wkv5_scan_matches_brute_force_and_explicit_sum():
+    T, H, S = 9, 3, 64
+    C = H * S
+    r, k, v = (rng.standard_normal((T, C)).astype(np.float32) for _ in range(3))
+    w = np.exp(-np.exp(rng.uniform(-6, 0, (H, S)))).astype(np.float32)
+    u = rng.uniform(-1, 1, (H, S)).astype(np.float32)
+    s0 = rng.standard_normal((H, S, S)).astype(np.float32)
+    y, s = po.wkv5_2_seq_f32(s0, r, k, v, w, u)
+    yb, sb = _wkv5_brute(*(a.astype(np.float64) for a in (r, k, v, w, u)), s0)
+    assert np.allclose(y, yb, rtol=1e-4, atol=1e-4)
+    assert np.allclose(s, sb, rtol=1e-4, atol=1e-4)
+    # S_T = diag(w)^T S_0 + sum_i diag(w)^(T-1-i) k_i v_i^T
+    for hd in range(H):
+        sl = slice(hd * S, (hd + 1) * S)
+        ex = (w[hd].astype(np.float64) ** T)[:, None] * s0[hd]
+        for i in range(T):
+            ex += (w[hd].astype(np.float64) ** (T - 1 - i))[:, None] * np.outer(k[i, sl], v[i, sl])
+        assert np.allclose(s[hd], ex, rtol=1e-4, atol=1e-4)
+
+
+# ---------------------------------------------------------------- dequant u8
+def _dequant_numpy(q, mx, rx, my, ry):
+    """Independent numpy-float16 statement of the dequantisation: every operation in
+    binary16; the fused multiply-add done exactly in float64 (exact for these operands)."""
+    c255 = (rx / np.float16(255)).astype(np.float16)
+    a = (c255[None, :] * ry[:, None]).astype(np.float16)
+    b = (mx[None, :] + my[:, None]).astype(np.float16)
+    # q*a has <= 19 significant bits and |exponent gap| to b is small: float64 sum is exact
+    exact = q.astype(np.float64) * a.astype(np.float64) + b.astype(np.float64)
+    return exact.astype(np.float16)  # float64 -> float16 in numpy is a single RTNE rounding
+
+
+def test_dequant_all_codes_times_scale_grid_bit_exact():
+    q = np.arange(256, dtype=np.uint8)[:, None].repeat(64, axis=1)  # K=256 rows: code = row index
+    mxs = h([-0.09, -0.031, 0.0, 0.0123, -1.7, 3e-5, -0.5, 2.0])
+    rxs = h([0.17, 0.011, 1.0, 0.33, 5.5, 1e-3, 0.0625, 2.5e-4])
+    N = 64
+    mx = np.tile(mxs, 8)
+    rx = np.repeat(rxs, 8)
+    for my_v, ry_v in [(-0.07, 0.93), (0.0, 1.0), (0.011, 0.5), (-2.0, 0.031), (6e-5, 0.999)]:
+        my = np.full(256, my_v, np.float16)
+        ry = np.full(256, ry_v, np.float16)
+        got = po.dequant_u8(q, mx, rx, my, ry)
+        ref = _dequant_numpy(q, mx, rx, my, ry)
+        assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+    # scalar entry point agrees with the matrix one
+    s = po.lib.orc_dequant_u8_scalar(200, int(mx[3].view(np.uint16)), int(rx[3].view(np.uint16)),
+                                     int(my[0].view(np.uint16)), int(ry[0].view(np.uint16)))
+    assert s == got[200, 3].view(np.uint16)
+    assert N == got.shape[1]
+
+
+def test_quantise_then_dequantise_error_is_half_a_step():
+    K, N = 192, 160
+    w = h(rng.standard_normal((K, N)) * 0.02)
+    q, mx, rx, my, ry = quantize_u8(w)
+    assert q.min() == 0 and q.max() == 255
+    wd = po.dequant_u8(q, mx, rx, my, ry).astype(np.float64)
+    step = rx.astype(np.float64)[None, :] * ry.astype(np.float64)[:, None] / 255
+    err = np.abs(wd - w.astype(np.float64))
+    assert (err <= 0.5 * step + 3e-4).all()  # half a step + binary16 rounding of a,b,w^
+    assert err.mean() < 0.3 * step.mean() + 1e-4
