@@ -1,0 +1,281 @@
+// Primitive operators of the `hip` device: the ones kernels/kernels.h names that are
+// not fused into the one-token kernels (layernorm, groupnorm, cast_dtype, fill_,
+// scalar_div_, vgather), weight preparation, and the greedy sampler's argmax.
+#include "device_utils.h"
+#include "frhip_internal.h"
+
+#pragma clang fp contract(off)
+
+namespace frhip {
+
+// ---- layernorm over rows: one workgroup (256 threads) per row ----------------
+// kernels/cuda/layer_norm.cu:101-130.  fp32 statistics (two passes over registers
+// or, for long rows, over memory), eps 1e-5.  binary16: the normalised value is
+// rounded to half before the affine, which is done in half (layer_norm.cu:60-69).
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_rows_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                             const T* __restrict__ beta, T* __restrict__ y, int cols) {
+  __shared__ float red[4];
+  const T* xr = x + (size_t)blockIdx.x * cols;
+  T* yr = y + (size_t)blockIdx.x * cols;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < cols; i += 256) s += (float)xr[i];
+  const float mean = block_sum<4>(s, red) / (float)cols;
+  float q = 0.f;
+  for (int i = threadIdx.x; i < cols; i += 256) {
+    float d = (float)xr[i] - mean;
+    q += d * d;
+  }
+  float var = block_sum<4>(q, red) / (float)cols;
+  var = var > 0.f ? var : 0.f;
+  const float inv = 1.0f / sqrtf(var + 1e-5f);
+  for (int i = threadIdx.x; i < cols; i += 256) {
+    float n = ((float)xr[i] - mean) * inv;
+    if constexpr (sizeof(T) == 2) {
+      yr[i] = ((T)n * gamma[i]) + beta[i];
+    } else {
+      yr[i] = n * gamma[i] + beta[i];
+    }
+  }
+}
+
+// ---- groupnorm, fp32: one wavefront per (row, group) -------------------------
+// kernels/cuda/group_norm.cu:322-357 (instances = rows*groups, eps 1e-5).
+__global__ __launch_bounds__(256) void groupnorm_f32_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                            const float* __restrict__ beta, float* __restrict__ y,
+                                                            int instances, int groups, int gs) {
+  const int inst = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (inst >= instances) return;  // whole wave exits together
+  const int lane = threadIdx.x & (kWave - 1);
+  const int g = inst % groups;
+  const float* xr = x + (size_t)inst * gs;
+  float* yr = y + (size_t)inst * gs;
+  float s = 0.f;
+  for (int i = lane; i < gs; i += kWave) s += xr[i];
+  const float mean = wave_sum(s) / (float)gs;
+  float q = 0.f;
+  for (int i = lane; i < gs; i += kWave) {
+    float d = xr[i] - mean;
+    q += d * d;
+  }
+  float var = wave_sum(q) / (float)gs;
+  var = var > 0.f ? var : 0.f;
+  const float inv = 1.0f / sqrtf(var + 1e-5f);
+  for (int i = lane; i < gs; i += kWave) yr[i] = (xr[i] - mean) * inv * gamma[g * gs + i] + beta[g * gs + i];
+}
+
+template <typename S, typename D>
+__global__ void cast_kernel(const S* __restrict__ src, D* __restrict__ dst, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = (D)src[i];
+}
+
+template <typename T>
+__global__ void fill_kernel(T* x, T v, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = v;
+}
+
+// kernels/cuda/element_wise.cu:8-12: x = x / half(val)
+__global__ void scalar_div_f16_kernel(h1* x, h1 d, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = (h1)((float)x[i] / (float)d);  // rounded fp32 quotient == rounded half quotient
+}
+
+__global__ void gather_rows_kernel(const unsigned char* __restrict__ table, const int32_t* __restrict__ ids,
+                                   unsigned char* __restrict__ out, int row_bytes) {
+  const u32x4* src = reinterpret_cast<const u32x4*>(table + (size_t)ids[blockIdx.x] * row_bytes);
+  u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)blockIdx.x * row_bytes);
+  for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x) dst[i] = src[i];
+}
+
+// [K][N] -> [N][K] through a 64x64 LDS tile (+1 padding against bank conflicts).
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst, int K, int N) {
+  __shared__ T tile[64][65];
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int r = ty; r < 64; r += 4) {
+    int k = k0 + r, n = n0 + tx;
+    if (k < K && n < N) tile[r][tx] = src[(size_t)k * N + n];
+  }
+  __syncthreads();
+  for (int r = ty; r < 64; r += 4) {
+    int n = n0 + r, k = k0 + tx;
+    if (k < K && n < N) dst[(size_t)n * K + k] = tile[tx][r];
+  }
+}
+
+// Packed uint8 [N][K] -> packed binary16 [N][K]; thread handles 4 codes of one row.
+__global__ void dequant_u8_kernel(const uint32_t* __restrict__ q, const h1* __restrict__ mx, const h1* __restrict__ rx,
+                                  const h1* __restrict__ my, const h1* __restrict__ ry, h4* __restrict__ out, int K,
+                                  int N) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // index of a 4-code word
+  const size_t words = (size_t)N * (K >> 2);
+  if (i >= words) return;
+  const int n = (int)(i / (K >> 2));
+  const int k = (int)(i % (K >> 2)) * 4;
+  const h1 c = dequant_c255(rx[n]);
+  const h2 c2 = {c, c};
+  const h2 m2 = {mx[n], mx[n]};
+  const uint32_t w = q[i];
+  h2 ry01 = {ry[k], ry[k + 1]}, ry23 = {ry[k + 2], ry[k + 3]};
+  h2 my01 = {my[k], my[k + 1]}, my23 = {my[k + 2], my[k + 3]};
+  h2 lo = dequant_pair<0>(w, c2, m2, ry01, my01);
+  h2 hi = dequant_pair<1>(w, c2, m2, ry23, my23);
+  out[i] = (h4){lo.x, lo.y, hi.x, hi.y};
+}
+
+// Index of the maximum, first occurrence on ties; single workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void argmax_f32_kernel(const float* __restrict__ x, int n, int32_t* out) {
+  __shared__ float bv[16];
+  __shared__ int bi[16];
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    float v = x[i];
+    if (v > best || (v == best && i < idx)) {
+      best = v;
+      idx = i;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    float ov = __shfl_xor(best, off);
+    int oi = __shfl_xor(idx, off);
+    if (ov > best || (ov == best && oi < idx)) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    bv[threadIdx.x >> 6] = best;
+    bi[threadIdx.x >> 6] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; w++)
+      if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
+        best = bv[w];
+        idx = bi[w];
+      }
+    *out = idx == 0x7fffffff ? 0 : idx;
+  }
+}
+
+}  // namespace frhip
+
+using namespace frhip;
+
+static unsigned blocks_for(size_t n, unsigned per) { return (unsigned)((n + per - 1) / per); }
+
+extern "C" {
+
+int frhip_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, int dtype,
+                    frhip_stream s) {
+  if (!x || !gamma || !beta || !y) return set_error(FRHIP_EINVAL, "layernorm: null pointer");
+  if (rows < 0 || cols <= 0) return set_error(FRHIP_ESHAPE, "layernorm: bad shape");
+  if (rows == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(s);
+  if (dtype == FRHIP_F16)
+    hipLaunchKernelGGL(layernorm_rows_kernel<h1>, dim3(rows), dim3(256), 0, st, (const h1*)x, (const h1*)gamma,
+                       (const h1*)beta, (h1*)y, cols);
+  else if (dtype == FRHIP_F32)
+    hipLaunchKernelGGL(layernorm_rows_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)x,
+                       (const float*)gamma, (const float*)beta, (float*)y, cols);
+  else
+    return set_error(FRHIP_EINVAL, "layernorm: dtype must be F16 or F32");
+  return check_launch("layernorm");
+}
+
+int frhip_groupnorm_f32(const float* x, int groups, const float* gamma, const float* beta, float* y, int rows,
+                        int cols, frhip_stream s) {
+  if (!x || !gamma || !beta || !y) return set_error(FRHIP_EINVAL, "groupnorm: null pointer");
+  if (rows < 0 || cols <= 0 || groups <= 0 || cols % groups != 0) return set_error(FRHIP_ESHAPE, "groupnorm: bad shape");
+  if (rows == 0) return 0;
+  const int inst = rows * groups;
+  hipLaunchKernelGGL(groupnorm_f32_kernel, dim3((inst + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(s), x, gamma,
+                     beta, y, inst, groups, cols / groups);
+  return check_launch("groupnorm");
+}
+
+int frhip_cast(const void* src, int sd, void* dst, int dd, size_t n, frhip_stream s) {
+  if (!src || !dst) return set_error(FRHIP_EINVAL, "cast: null pointer");
+  if (n == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(s);
+  if (sd == FRHIP_F16 && dd == FRHIP_F32)
+    hipLaunchKernelGGL((cast_kernel<h1, float>), dim3(blocks_for(n, 256)), dim3(256), 0, st, (const h1*)src, (float*)dst, n);
+  else if (sd == FRHIP_F32 && dd == FRHIP_F16)
+    hipLaunchKernelGGL((cast_kernel<float, h1>), dim3(blocks_for(n, 256)), dim3(256), 0, st, (const float*)src, (h1*)dst, n);
+  else if (sd == dd && (sd == FRHIP_F16 || sd == FRHIP_F32))
+    return hip_result(hipMemcpyAsync(dst, src, n * (sd == FRHIP_F16 ? 2 : 4), hipMemcpyDeviceToDevice, st), "cast copy");
+  else
+    return set_error(FRHIP_EINVAL, "cast: unsupported dtype pair");
+  return check_launch("cast");
+}
+
+int frhip_fill(void* x, int dtype, float value, size_t n, frhip_stream s) {
+  if (!x) return set_error(FRHIP_EINVAL, "fill: null pointer");
+  if (n == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(s);
+  if (dtype == FRHIP_F16)
+    hipLaunchKernelGGL(fill_kernel<h1>, dim3(blocks_for(n, 256)), dim3(256), 0, st, (h1*)x, (h1)value, n);
+  else if (dtype == FRHIP_F32)
+    hipLaunchKernelGGL(fill_kernel<float>, dim3(blocks_for(n, 256)), dim3(256), 0, st, (float*)x, value, n);
+  else if (dtype == FRHIP_U8)
+    hipLaunchKernelGGL(fill_kernel<unsigned char>, dim3(blocks_for(n, 256)), dim3(256), 0, st, (unsigned char*)x,
+                       (unsigned char)value, n);
+  else
+    return set_error(FRHIP_EINVAL, "fill: unknown dtype");
+  return check_launch("fill");
+}
+
+int frhip_scalar_div_f16(void* x, float divisor, size_t n, frhip_stream s) {
+  if (!x) return set_error(FRHIP_EINVAL, "scalar_div: null pointer");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(scalar_div_f16_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, static_cast<hipStream_t>(s), (h1*)x,
+                     (h1)divisor, n);
+  return check_launch("scalar_div");
+}
+
+int frhip_gather_rows(const void* table, const int32_t* ids_dev, void* out, int n_ids, int row_bytes, frhip_stream s) {
+  if (!table || !ids_dev || !out) return set_error(FRHIP_EINVAL, "gather: null pointer");
+  if (n_ids < 0 || row_bytes <= 0 || row_bytes % 16 != 0) return set_error(FRHIP_ESHAPE, "gather: row_bytes must be a multiple of 16");
+  if (n_ids == 0) return 0;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(n_ids), dim3(256), 0, static_cast<hipStream_t>(s),
+                     (const unsigned char*)table, ids_dev, (unsigned char*)out, row_bytes);
+  return check_launch("gather_rows");
+}
+
+int frhip_pack_transpose(const void* src, void* dst, int K, int N, int elem_bytes, frhip_stream s) {
+  if (!src || !dst) return set_error(FRHIP_EINVAL, "pack: null pointer");
+  if (K <= 0 || N <= 0) return set_error(FRHIP_ESHAPE, "pack: empty matrix");
+  dim3 grid((N + 63) / 64, (K + 63) / 64);
+  hipStream_t st = static_cast<hipStream_t>(s);
+  if (elem_bytes == 2)
+    hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t*)src, (uint16_t*)dst, K, N);
+  else if (elem_bytes == 1)
+    hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, st, (const uint8_t*)src, (uint8_t*)dst, K, N);
+  else
+    return set_error(FRHIP_EINVAL, "pack: elem_bytes must be 1 or 2");
+  return check_launch("pack_transpose");
+}
+
+int frhip_dequant_u8(const frhip_weight* w, void* dst, frhip_stream s) {
+  if (!w || !w->data || !dst) return set_error(FRHIP_EINVAL, "dequant: null pointer");
+  if (w->dtype != FRHIP_U8 || !w->mx || !w->rx || !w->my || !w->ry) return set_error(FRHIP_EINVAL, "dequant: not a uint8 weight");
+  if (w->K <= 0 || w->N <= 0 || w->K % 4 != 0) return set_error(FRHIP_ESHAPE, "dequant: K must be a multiple of 4");
+  const size_t words = (size_t)w->N * (w->K / 4);
+  hipLaunchKernelGGL(dequant_u8_kernel, dim3(blocks_for(words, 256)), dim3(256), 0, static_cast<hipStream_t>(s),
+                     (const uint32_t*)w->data, (const h1*)w->mx, (const h1*)w->rx, (const h1*)w->my, (const h1*)w->ry,
+                     (h4*)dst, w->K, w->N);
+  return check_launch("dequant_u8");
+}
+
+int frhip_argmax_f32(const float* logits, int n, int32_t* out_id, frhip_stream s) {
+  if (!logits || !out_id) return set_error(FRHIP_EINVAL, "argmax: null pointer");
+  if (n <= 0) return set_error(FRHIP_ESHAPE, "argmax: empty input");
+  hipLaunchKernelGGL(argmax_f32_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(s), logits, n, out_id);
+  return check_launch("argmax");
+}
+
+}  // extern "C"

@@ -1,0 +1,161 @@
+/*
+ * frhip.h -- C ABI of the MI355X (gfx950) RWKV inference kernels.
+ *
+ * This is the boundary a faster-rwkv `hip` device binds to: the host-side operator
+ * functions registered in kernels/registry.h for Device::kHIP call nothing but these
+ * entry points.  Plain pointers and sizes only; no C++ or HIP types cross it.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t value when the HIP
+ *     runtime failed, or a negative FRHIP_E* value when the arguments are rejected
+ *     before anything is launched.  Nothing throws.  frhip_error_string() describes
+ *     the most recent failure of the calling thread.
+ *   - `stream` is an opaque handle from frhip_stream_create(), or NULL for the
+ *     default (null) stream.  All launches are asynchronous with respect to the host.
+ *   - device pointers are plain `void *`; binary16 data is IEEE half, "f32" is float.
+ *   - activations are vectors [C] (one token) or row-major [T, C] (seq mode).
+ *   - matrix weights are held on the device OUTPUT-MAJOR: element (k, n) of the
+ *     reference's row-major [K=in, N=out] tensor (tools/convert_weight.py:44-46,
+ *     kernels/cuda/matmul.cpp:105-121) lives at data[n*K + k].  frhip_pack_* produce
+ *     that layout from the reference's.  A wavefront then streams whole rows of K
+ *     contiguous elements and reduces them with cross-lane adds, and the prefill
+ *     GEMM reads both operands K-contiguous.
+ */
+#ifndef FRHIP_H_
+#define FRHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FRHIP_ABI_VERSION 1
+
+enum {
+  FRHIP_EINVAL = -1,  /* bad argument (null pointer, negative size, unknown enum) */
+  FRHIP_ESHAPE = -2,  /* shape not supported by the kernel (alignment, maximum)  */
+  FRHIP_ESTATE = -3,  /* call not valid now (e.g. graph capture not in progress)  */
+  FRHIP_ENODEV = -4   /* no usable gfx950 device                                  */
+};
+
+enum { FRHIP_F32 = 0, FRHIP_F16 = 1, FRHIP_U8 = 2 };
+enum { FRHIP_H2D = 0, FRHIP_D2H = 1, FRHIP_D2D = 2 };
+
+typedef void *frhip_stream;
+typedef void *frhip_event;
+typedef void *frhip_graph;
+
+/* A matrix weight as the kernels consume it.  For FRHIP_U8 the ChatRWKV-style
+ * per-column (mx, rx: [N]) and per-row (my, ry: [K]) binary16 offsets and ranges
+ * accompany the codes (parameters named at kernels/kernels.h:11-13); for FRHIP_F16
+ * they are NULL. */
+typedef struct frhip_weight {
+  const void *data; /* [N][K] output-major, binary16 or uint8 */
+  const void *mx, *rx; /* [N] binary16 */
+  const void *my, *ry; /* [K] binary16 */
+  int32_t K, N;
+  int32_t dtype; /* FRHIP_F16 or FRHIP_U8 */
+} frhip_weight;
+
+/* ---- runtime: replaces the cudart calls of tensor.cpp:58-96 and the raw
+ *      cudaMalloc/cudaFree under kernels/cuda/allocator.cpp:412-460 ------------- */
+int frhip_abi_version(void);
+const char *frhip_error_string(void);
+int frhip_device_count(int *count);
+int frhip_init(int device);                         /* select device, create handles */
+int frhip_device_info(char *name, size_t name_len, int *compute_units, size_t *total_mem);
+int frhip_malloc(void **ptr, size_t bytes);         /* hipMalloc; caching sits above, in the host allocator */
+int frhip_free(void *ptr);
+int frhip_host_malloc(void **ptr, size_t bytes);    /* pinned host memory for logits read-back */
+int frhip_host_free(void *ptr);
+int frhip_memcpy(void *dst, const void *src, size_t bytes, int kind);              /* blocking, as cudaMemcpy at tensor.cpp:65-73 */
+int frhip_memcpy_async(void *dst, const void *src, size_t bytes, int kind, frhip_stream s);
+int frhip_memset_async(void *dst, int byte, size_t bytes, frhip_stream s);
+int frhip_stream_create(frhip_stream *s);
+int frhip_stream_destroy(frhip_stream s);
+int frhip_stream_sync(frhip_stream s);
+int frhip_device_sync(void);
+int frhip_event_create(frhip_event *e);
+int frhip_event_destroy(frhip_event e);
+int frhip_event_record(frhip_event e, frhip_stream s);
+int frhip_event_sync(frhip_event e);
+int frhip_event_elapsed_ms(frhip_event start, frhip_event stop, float *ms);
+/* Capture everything launched on `s` between begin and end into a replayable graph
+ * (the reference issues ~415 launches per token, kernels/default/model_forward.cpp:105-188). */
+int frhip_graph_begin(frhip_stream s);
+int frhip_graph_end(frhip_stream s, frhip_graph *g);
+int frhip_graph_launch(frhip_graph g, frhip_stream s);
+int frhip_graph_destroy(frhip_graph g);
+
+/* ---- weight preparation ---------------------------------------------------- */
+/* src: the reference's [K][N] row-major matrix on the device; dst: [N][K].
+ * elem_bytes 1 (uint8 codes) or 2 (binary16). */
+int frhip_pack_transpose(const void *src_kn, void *dst_nk, int K, int N, int elem_bytes, frhip_stream s);
+/* Dequantise a packed uint8 weight into packed binary16, dst [N][K].  Every
+ * operation in binary16, round-to-nearest-even:
+ *   c = rx[n] / 255;  a = c * ry[k];  b = mx[n] + my[k];  w^ = fma(q, a, b). */
+int frhip_dequant_u8(const frhip_weight *w, void *dst_nk_f16, frhip_stream s);
+
+/* ---- primitive operators (names of kernels/kernels.h) ------------------------ */
+/* layernorm: kernels/cuda/layer_norm.cu:101-130.  dtype FRHIP_F16 or FRHIP_F32 for x, gamma, beta, y. */
+int frhip_layernorm(const void *x, const void *gamma, const void *beta, void *y, int rows, int cols, int dtype, frhip_stream s);
+/* groupnorm over fp32 rows: kernels/cuda/group_norm.cu:322-357. */
+int frhip_groupnorm_f32(const float *x, int groups, const float *gamma, const float *beta, float *y, int rows, int cols, frhip_stream s);
+/* matmul, vector x matrix: kernels/cuda/matmul.cpp:105-109.  x [K] binary16; y [N] in out_dtype (F16 or F32). */
+int frhip_gemv(const void *x, const frhip_weight *w, void *y, int out_dtype, frhip_stream s);
+/* cast_dtype: kernels/cuda/cast_dtype.cu:24-41. */
+int frhip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n, frhip_stream s);
+/* fill_: kernels/cuda/fill.cu:17-27. */
+int frhip_fill(void *x, int dtype, float value, size_t n, frhip_stream s);
+/* scalar_div_: kernels/cuda/element_wise.cu:8-19 (binary16, divisor rounded to half first). */
+int frhip_scalar_div_f16(void *x, float divisor, size_t n, frhip_stream s);
+/* vgather of embedding rows: kernels/default/gather_ops.cpp:46-89.  table [V][C]; ids on the device. */
+int frhip_gather_rows(const void *table, const int32_t *ids_dev, void *out, int n_ids, int row_bytes, frhip_stream s);
+
+/* ---- fused one-token operators ------------------------------------------------ */
+/* Scratch the fused operators need: frhip_decode_workspace_bytes(C, F) bytes,
+ * 256-byte aligned, owned by the caller, reusable across calls on one stream. */
+size_t frhip_decode_workspace_bytes(int C, int F);
+
+/* att (RWKV-4, one token): kernels/cuda/att.cu:182-217,337-359.
+ * Reads x, sx [C] binary16; aa, bb, pp [C] fp32; writes x_out = x + out, xx_out =
+ * LN(x) (the new shift state), aa_out, bb_out, pp_out.  aa_out/bb_out/pp_out may
+ * alias aa/bb/pp and x_out may alias x; xx_out must not alias sx. */
+int frhip_att_one_v4(int C, const void *x, const void *sx, const float *aa, const float *bb, const float *pp,
+                     const void *ln_w, const void *ln_b, const void *k_mix, const void *v_mix, const void *r_mix,
+                     const float *t_decay, const float *t_first,
+                     const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw, const frhip_weight *ow,
+                     void *x_out, void *xx_out, float *aa_out, float *bb_out, float *pp_out,
+                     void *workspace, frhip_stream s);
+
+/* ffn (one token): kernels/cuda/ffn.cu:62-110.  post_div2 != 0 additionally applies the
+ * x /= 2 rescale of kernels/default/model_forward.cpp:173-175 to x_out. */
+int frhip_ffn_one(int C, int F, const void *x, const void *sx, const void *ln_w, const void *ln_b,
+                  const void *k_mix, const void *r_mix,
+                  const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                  void *x_out, void *xx_out, int post_div2, void *workspace, frhip_stream s);
+
+/* layernorm(ln_out) -> head matmul -> cast to fp32: kernels/default/model_forward.cpp:180-188. */
+int frhip_head(int C, const void *x, const void *ln_w, const void *ln_b, const frhip_weight *head, float *logits, frhip_stream s);
+
+/* att_one_v5_1 (RWKV-5.1/5.2, one token): kernels/cuda/att.cu:267-335,393-425.
+ * s [H][S][S] fp32 ([head][key][value]); t_decay, t_first [H][S]; lx_w, lx_b [C] fp32.
+ * s_out may alias s. */
+int frhip_att_one_v5_1(int C, int H, const void *x, const void *sx, const float *s,
+                       const void *ln_w, const void *ln_b, const float *lx_w, const float *lx_b,
+                       const void *k_mix, const void *v_mix, const void *r_mix, const void *g_mix,
+                       const float *t_decay, const float *t_first,
+                       const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                       const frhip_weight *gw, const frhip_weight *ow,
+                       void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
+
+/* greedy sampler step (Sampler::Sample with top_k = 1, chat.cpp:76-77): index of the
+ * largest logit, first one on ties, written to *out_id on the device. */
+int frhip_argmax_f32(const float *logits, int n, int32_t *out_id, frhip_stream s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FRHIP_H_ */

@@ -1,0 +1,112 @@
+"""Test-side helpers: drive the HIP kernels through the C ABI (ctypes) on numpy data."""
+import ctypes as C
+import importlib
+
+import numpy as np
+
+fr = importlib.import_module("faster-rwkv_amd")
+DevBuf, PackedWeight = fr.DevBuf, fr.PackedWeight
+
+
+def L():
+    return fr.lib()
+
+
+def dev(a):
+    return DevBuf.from_numpy(a)
+
+
+def ulp_diff_f16(a, b):
+    """Distance in units of binary16 representable values (monotone integer mapping)."""
+    def key(x):
+        u = np.asarray(x, np.float16).view(np.uint16).astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(key(a) - key(b))
+
+
+def assert_close_f16(got, ref, max_ulp=2, max_frac=0.03, what=""):
+    """|got-ref| <= max_ulp binary16 spacings, the spacing taken at max(|ref|, rms(ref)/4):
+    an output formed by cancellation (x + out close to 0) inherits the absolute rounding
+    error of its operands, which is not small in units of its own tiny spacing."""
+    got, ref = np.asarray(got, np.float16), np.asarray(ref, np.float16)
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    g32, r32 = got.astype(np.float32), ref.astype(np.float32)
+    assert np.isfinite(g32).all(), what + ": non-finite output"
+    floor = 0.25 * float(np.sqrt(np.mean(r32.astype(np.float64) ** 2))) + 1e-6
+    mag = np.maximum(np.abs(r32), floor)
+    spacing = np.exp2(np.floor(np.log2(mag)) - 10)
+    err = np.abs(g32 - r32)
+    bad = err > max_ulp * spacing
+    assert not bad.any(), "%s: %d elements beyond %d spacings (worst %.2f)" % (
+        what, bad.sum(), max_ulp, float((err / spacing).max()))
+    assert (got.view(np.uint16) != ref.view(np.uint16)).mean() <= max_frac, "%s: %.3f of elements differ" % (
+        what, (got.view(np.uint16) != ref.view(np.uint16)).mean())
+
+
+def make_weight(w_kn, quant=False):
+    """PackedWeight from a [K,N] half matrix; quant=True quantises to uint8 first and
+    also returns the oracle's dequantised [K,N] half matrix."""
+    if not quant:
+        return PackedWeight(w_kn=w_kn), np.ascontiguousarray(w_kn, np.float16)
+    import pyoracle as po
+    from synth import quantize_u8
+    q, mx, rx, my, ry = quantize_u8(w_kn)
+    return PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry), po.dequant_u8(q, mx, rx, my, ry)
+
+
+class HipModelV4:
+    """RWKV-4 one-token forward assembled from the fused C-ABI operators, in the order of
+    kernels/default/model_forward.cpp:105-188.  Parameters in the reference's positional order."""
+
+    def __init__(self, L_, C_, F_, V_, params, emb, quant=False):
+        self.L, self.C, self.F, self.V = L_, C_, F_, V_
+        self.mats = {}
+        self.oracle_params = list(params)
+        self.p = []
+        mat_pos = set()
+        for l in range(L_):
+            mat_pos |= {l * 18 + j for j in (7, 8, 9, 10, 15, 16, 17)}
+        mat_pos.add(L_ * 18 + 2)
+        for i, a in enumerate(params):
+            if i in mat_pos:
+                w, deq = make_weight(a, quant)
+                self.p.append(w)
+                self.oracle_params[i] = deq
+            else:
+                self.p.append(dev(a))
+        self.emb = dev(emb)
+        self.emb_np = emb
+        self.ws = DevBuf(L().frhip_decode_workspace_bytes(C_, F_))
+        self.x = [DevBuf.empty(C_, np.float16) for _ in range(2)]
+        self.logits = DevBuf.empty(V_, np.float32)
+        self.reset()
+
+    def reset(self):
+        C_ = self.C
+        self.state = []
+        for _ in range(self.L):
+            self.state.append([dev(np.zeros(C_, np.float16)), dev(np.zeros(C_, np.float32)),
+                               dev(np.zeros(C_, np.float32)), dev(np.full(C_, -1e30, np.float32)),
+                               dev(np.zeros(C_, np.float16))])
+        self.spare = [dev(np.zeros(C_, np.float16)), dev(np.zeros(C_, np.float16))]
+
+    def run(self, tok):
+        lib, C_, F_ = L(), self.C, self.F
+        fr.check(lib.frhip_memcpy(self.x[0].ptr, self.emb.ptr + int(tok) * C_ * 2, C_ * 2, fr.D2D))
+        x = self.x[0]
+        for l in range(self.L):
+            p = self.p[l * 18:(l + 1) * 18]
+            st = self.state[l]
+            fr.check(lib.frhip_att_one_v4(C_, x.ptr, st[0].ptr, st[1].ptr, st[2].ptr, st[3].ptr,
+                                          p[0].ptr, p[1].ptr, p[2].ptr, p[3].ptr, p[4].ptr, p[5].ptr, p[6].ptr,
+                                          p[7].ref, p[8].ref, p[9].ref, p[10].ref,
+                                          x.ptr, self.spare[0].ptr, st[1].ptr, st[2].ptr, st[3].ptr,
+                                          self.ws.ptr, None), "att")
+            st[0], self.spare[0] = self.spare[0], st[0]
+            fr.check(lib.frhip_ffn_one(C_, F_, x.ptr, st[4].ptr, p[11].ptr, p[12].ptr, p[13].ptr, p[14].ptr,
+                                       p[15].ref, p[16].ref, p[17].ref, x.ptr, self.spare[1].ptr,
+                                       1 if (l + 1) % 6 == 0 else 0, self.ws.ptr, None), "ffn")
+            st[4], self.spare[1] = self.spare[1], st[4]
+        t = self.p[self.L * 18:]
+        fr.check(lib.frhip_head(C_, x.ptr, t[0].ptr, t[1].ptr, t[2].ref, self.logits.ptr, None), "head")
+        return self.logits.numpy()

@@ -1,0 +1,163 @@
+"""GPU parity tests of the primitive operators, through the C ABI, against the oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import pyoracle as po
+from hipref import DevBuf, L, PackedWeight, assert_close_f16, dev, fr, make_weight
+
+_alive = []
+
+
+def keep(a):
+    """Upload and keep the buffer alive until the test module is torn down (a temporary
+    DevBuf would be freed as soon as its .ptr has been read)."""
+    b = dev(a)
+    _alive.append(b)
+    if len(_alive) > 64:
+        fr.check(L().frhip_device_sync())
+        del _alive[:32]
+    return b
+
+
+rng = np.random.default_rng(123)
+
+
+def h(x):
+    return np.asarray(x, np.float32).astype(np.float16)
+
+
+def test_runtime_identifies_gfx950_and_roundtrips_memory():
+    fr.init()
+    name = C.create_string_buffer(128)
+    cus, mem = C.c_int(), C.c_size_t()
+    fr.check(L().frhip_device_info(name, 128, C.byref(cus), C.byref(mem)))
+    print("device:", name.value.decode(), cus.value, "CUs", mem.value >> 30, "GiB", flush=True)
+    assert b"gfx950" in name.value and cus.value >= 200
+    a = rng.integers(0, 255, 100003).astype(np.uint8)
+    assert np.array_equal(keep(a).numpy(), a)
+
+
+def test_known_answer_fill_then_scalar_div():
+    """tests/test_ops.cpp:9-16"""
+    x = DevBuf.empty(256, np.float16)
+    fr.check(L().frhip_fill(x.ptr, fr.F16, 1.0, 256, None))
+    fr.check(L().frhip_scalar_div_f16(x.ptr, 2.0, 256, None))
+    y = DevBuf.empty(256, np.float32)
+    fr.check(L().frhip_cast(x.ptr, fr.F16, y.ptr, fr.F32, 256, None))
+    assert (y.numpy() == np.float32(0.5)).all()
+
+
+@pytest.mark.parametrize("K,N,dt", [(64, 64, np.float16), (130, 70, np.float16), (257, 1000, np.uint8), (2048, 512, np.uint8)])
+def test_pack_transpose(K, N, dt):
+    a = rng.integers(0, 60000 if dt == np.float16 else 255, (K, N)).astype(np.uint16 if dt == np.float16 else np.uint8)
+    src, dst = keep(a), DevBuf.empty((N, K), a.dtype)
+    fr.check(L().frhip_pack_transpose(src.ptr, dst.ptr, K, N, a.dtype.itemsize, None))
+    assert np.array_equal(dst.numpy(), a.T)
+
+
+def test_cast_roundtrip_and_rtne():
+    x = (rng.standard_normal(5000) * 10).astype(np.float32)
+    a, b = keep(x), DevBuf.empty(5000, np.float16)
+    fr.check(L().frhip_cast(a.ptr, fr.F32, b.ptr, fr.F16, 5000, None))
+    assert np.array_equal(b.numpy().view(np.uint16), po.f2h(x).view(np.uint16))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 2048), (7, 768), (3, 2560), (33, 96)])
+def test_layernorm_f16(rows, cols):
+    x, g, b = h(rng.standard_normal((rows, cols)) * 3), h(1 + 0.1 * rng.standard_normal(cols)), h(0.1 * rng.standard_normal(cols))
+    y = DevBuf.empty((rows, cols), np.float16)
+    fr.check(L().frhip_layernorm(keep(x).ptr, keep(g).ptr, keep(b).ptr, y.ptr, rows, cols, fr.F16, None))
+    assert_close_f16(y.numpy(), po.layernorm_f16(x, g, b), max_ulp=1, what="layernorm")
+
+
+def test_layernorm_f32_and_groupnorm():
+    x = rng.standard_normal((5, 2560)).astype(np.float32)
+    g, b = rng.standard_normal(2560).astype(np.float32), rng.standard_normal(2560).astype(np.float32)
+    y = DevBuf.empty((5, 2560), np.float32)
+    fr.check(L().frhip_layernorm(keep(x).ptr, keep(g).ptr, keep(b).ptr, y.ptr, 5, 2560, fr.F32, None))
+    assert np.allclose(y.numpy(), po.layernorm_f32(x, g, b), atol=2e-5, rtol=1e-5)
+    fr.check(L().frhip_groupnorm_f32(keep(x).ptr, 40, keep(g).ptr, keep(b).ptr, y.ptr, 5, 2560, None))
+    assert np.allclose(y.numpy(), po.groupnorm_f32(x, 40, g, b), atol=2e-5, rtol=1e-5)
+
+
+def test_dequant_all_codes_bit_exact():
+    """Every code 0..255 against a grid of binary16 scale patterns, bit for bit."""
+    K, N = 256, 64
+    q = np.arange(256, dtype=np.uint8)[:, None].repeat(N, axis=1)
+    mxs = h([-0.09, -0.031, 0.0, 0.0123, -1.7, 3e-5, -0.5, 2.0])
+    rxs = h([0.17, 0.011, 1.0, 0.33, 5.5, 1e-3, 0.0625, 2.5e-4])
+    mx, rx = np.tile(mxs, 8), np.repeat(rxs, 8)
+    for my_v, ry_v in [(-0.07, 0.93), (0.0, 1.0), (0.011, 0.5), (-2.0, 0.031), (6e-5, 0.999)]:
+        my, ry = np.full(K, my_v, np.float16), np.full(K, ry_v, np.float16)
+        ref = po.dequant_u8(q, mx, rx, my, ry)  # [K,N]
+        w = PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry)
+        out = DevBuf.empty((N, K), np.float16)
+        fr.check(L().frhip_dequant_u8(w.ref, out.ptr, None))
+        assert np.array_equal(out.numpy().T.view(np.uint16), ref.view(np.uint16))
+        # the dequantisation fused into the matrix-vector kernel: a one-hot activation
+        # returns row k of the dequantised matrix exactly (fp32 output, 1*w + 0's)
+        y = DevBuf.empty(N, np.float32)
+        for k in (0, 1, 17, 200, 255):
+            e = np.zeros(K, np.float16)
+            e[k] = 1
+            fr.check(L().frhip_gemv(keep(e).ptr, w.ref, y.ptr, fr.F32, None))
+            assert np.array_equal(y.numpy(), ref[k].astype(np.float32)), k
+
+
+def test_dequant_random_matrix_bit_exact():
+    from synth import quantize_u8
+    K, N = 2048, 320
+    w = h(rng.standard_normal((K, N)) * 0.02)
+    q, mx, rx, my, ry = quantize_u8(w)
+    pw = PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry)
+    out = DevBuf.empty((N, K), np.float16)
+    fr.check(L().frhip_dequant_u8(pw.ref, out.ptr, None))
+    assert np.array_equal(out.numpy().T.view(np.uint16), po.dequant_u8(q, mx, rx, my, ry).view(np.uint16))
+
+
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 8192), (8192, 2048), (2560, 2560), (8960, 2560), (768, 50277), (64, 3), (16, 1)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_gemv_against_oracle(K, N, quant):
+    if quant and N > 20000:
+        pytest.skip("quantising a 50277-column matrix in numpy is slow; covered by the fp16 case")
+    x = h(rng.standard_normal(K))
+    w = h(rng.standard_normal((K, N)) * 0.02)
+    pw, wref = make_weight(w, quant)
+    ref32 = po.gemm_f16(x, wref, "f32")
+    y32, y16 = DevBuf.empty(N, np.float32), DevBuf.empty(N, np.float16)
+    fr.check(L().frhip_gemv(keep(x).ptr, pw.ref, y32.ptr, fr.F32, None))
+    fr.check(L().frhip_gemv(keep(x).ptr, pw.ref, y16.ptr, fr.F16, None))
+    tol = 2e-6 * np.sqrt(K) * np.abs(ref32).max() + 1e-6
+    assert np.abs(y32.numpy() - ref32).max() <= tol + 2e-5
+    assert_close_f16(y16.numpy(), ref32.astype(np.float16), max_ulp=1, what="gemv f16 out")
+
+
+def test_gemv_rejects_bad_arguments():
+    w = PackedWeight(w_kn=h(rng.standard_normal((64, 8))))
+    y = DevBuf.empty(8, np.float32)
+    x = keep(h(np.zeros(64)))
+    assert L().frhip_gemv(None, w.ref, y.ptr, fr.F32, None) == -1
+    assert L().frhip_gemv(x.ptr, w.ref, y.ptr, 7, None) == -1
+    bad = fr.Weight(w.c.data, None, None, None, None, 60, 8, fr.F16)
+    assert L().frhip_gemv(x.ptr, C.byref(bad), y.ptr, fr.F32, None) == -2
+    assert b"multiple of 16" in L().frhip_error_string()
+
+
+def test_argmax_first_of_ties():
+    x = rng.standard_normal(65536).astype(np.float32)
+    x[[1234, 40000]] = 9.0
+    out = DevBuf.empty(1, np.int32)
+    fr.check(L().frhip_argmax_f32(keep(x).ptr, 65536, out.ptr, None))
+    assert out.numpy()[0] == 1234 == po.lib.orc_argmax(x.ctypes.data_as(C.c_void_p), 65536)
+
+
+def test_gather_rows():
+    tab = h(rng.standard_normal((1000, 256)))
+    ids = np.array([5, 999, 0, 5, 123], np.int32)
+    out = DevBuf.empty((5, 256), np.float16)
+    fr.check(L().frhip_gather_rows(keep(tab).ptr, keep(ids).ptr, out.ptr, 5, 512, None))
+    assert np.array_equal(out.numpy(), tab[ids])
