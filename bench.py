@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batch-1 greedy decode of an RWKV-4 1.5B-shaped model on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 512] [--warmup 16] [--dtype fp16|int8]
+
+A "step" is one decoded token: rwkv::Model::Run(id) through the `hip` device (fused kernels
+replayed as a HIP graph), the fp32 logits copied to the host, and the host-side argmax that
+picks the next token -- the loop chat.cpp runs with top_k = 1.  Weights are random-init of
+the named architecture (there are no checkpoints here) and are resident in HBM before the
+timed region starts.
+
+Prints ONE JSON line.  Besides the decode rate it carries
+  roofline     -- the row-streaming matrix-vector kernels (all of their launches in one
+                  token): algorithmic bytes / summed launch time, measured with HIP events on
+                  the launch stream, against the 8 TB/s HBM peak;
+  cpu_baseline -- the CPU oracle's fp32 path (oracle/, a port: the reference has no CPU model
+                  path) timed on this host on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "oracle")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+
+CONFIGS = {
+    # BASELINE.json configs[1] / configs[2]
+    "fp16": dict(workload="rwkv4-1.5B-shaped fp16 decode bs1 (24 layers, d_model 2048, ffn 8192, vocab 65536)",
+                 spec="synthetic:v=4,L=24,C=2048,F=8192,V=65536,seed=1236", strategy="hip fp16", wbytes=2),
+    "int8": dict(workload="rwkv4-1.5B-shaped uint8 decode bs1 (24 layers, d_model 2048, ffn 8192, vocab 65536)",
+                 spec="synthetic:v=4,L=24,C=2048,F=8192,V=65536,seed=1237", strategy="hip int8", wbytes=1),
+}
+L_, C_, F_, V_ = 24, 2048, 8192, 65536
+
+
+def algorithmic_bytes_per_token(wbytes):
+    """Bytes the matrix-vector kernels must move per token: every matrix weight once, plus
+    (uint8) its offsets/ranges, plus the activation vector in and the result out."""
+    mats = [(C_, C_)] * 4 + [(C_, F_), (F_, C_), (C_, C_)]
+    per_layer = 0
+    for k, n in mats:
+        per_layer += k * n * wbytes + 2 * k + 2 * n
+        if wbytes == 1:
+            per_layer += 4 * (k + n)
+    head = C_ * V_ * wbytes + 2 * C_ + 4 * V_ + (4 * (C_ + V_) if wbytes == 1 else 0)
+    return L_ * per_layer + head
+
+
+def measure_kernels(fr, cfg, reps=20):
+    """Time the launches of one token with HIP events recorded on the launch stream itself:
+    total time of the fused kernels (they are back to back on one stream, so the events
+    bracket exactly their execution), averaged over `reps` tokens after a warm-up."""
+    lib = fr.lib()
+    fr.init()
+    rng = np.random.default_rng(0)
+    u8 = cfg["wbytes"] == 1
+    keep = []
+
+    def dev(a):
+        b = fr.DevBuf.from_numpy(a)
+        keep.append(b)
+        return b
+
+    def weight(K, N):
+        if u8:
+            d = dev(rng.integers(0, 255, (N, K), dtype=np.uint8))
+            sc = [dev(rng.uniform(0.01, 0.02, n).astype(np.float16)) for n in (N, N, K, K)]
+            return fr.Weight(d.ptr, sc[0].ptr, sc[1].ptr, sc[2].ptr, sc[3].ptr, K, N, fr.U8)
+        d = dev((rng.standard_normal((N, K), dtype=np.float32) * 0.02).astype(np.float16))
+        return fr.Weight(d.ptr, None, None, None, None, K, N, fr.F16)
+
+    h = lambda a: np.asarray(a, np.float32).astype(np.float16)
+    layers = []
+    for _ in range(L_):
+        layers.append(dict(
+            vec=[dev(h(np.ones(C_))), dev(h(np.zeros(C_))), dev(h(rng.uniform(0, 1, C_))), dev(h(rng.uniform(0, 1, C_))),
+                 dev(h(rng.uniform(0, 1, C_)))],
+            td=dev((-np.exp(rng.uniform(-5, 1, C_))).astype(np.float32)), tf=dev(rng.uniform(-1, 1, C_).astype(np.float32)),
+            att=[weight(C_, C_) for _ in range(4)],
+            fvec=[dev(h(np.ones(C_))), dev(h(np.zeros(C_))), dev(h(rng.uniform(0, 1, C_))), dev(h(rng.uniform(0, 1, C_)))],
+            ffn=[weight(C_, F_), weight(F_, C_), weight(C_, C_)],
+            st=[dev(h(np.zeros(C_))), dev(np.zeros(C_, np.float32)), dev(np.zeros(C_, np.float32)),
+                dev(np.full(C_, -1e30, np.float32)), dev(h(np.zeros(C_)))],
+            xx=[dev(h(np.zeros(C_))), dev(h(np.zeros(C_)))]))
+    ln_o = [dev(h(np.ones(C_))), dev(h(np.zeros(C_)))]
+    head = weight(C_, V_)
+    x = dev(h(rng.standard_normal(C_)))
+    logits = fr.DevBuf.empty(V_, np.float32)
+    ws = fr.DevBuf(lib.frhip_decode_workspace_bytes(C_, F_))
+    st = C.c_void_p()
+    fr.check(lib.frhip_stream_create(C.byref(st)))
+
+    def token():
+        for l, v in enumerate(layers):
+            s = v["st"]
+            fr.check(lib.frhip_att_one_v4(C_, x.ptr, s[0].ptr, s[1].ptr, s[2].ptr, s[3].ptr, *[t.ptr for t in v["vec"]],
+                                          v["td"].ptr, v["tf"].ptr, *[C.byref(w) for w in v["att"]], x.ptr,
+                                          v["xx"][0].ptr, s[1].ptr, s[2].ptr, s[3].ptr, ws.ptr, st))
+            fr.check(lib.frhip_ffn_one(C_, F_, x.ptr, s[4].ptr, *[t.ptr for t in v["fvec"]],
+                                       *[C.byref(w) for w in v["ffn"]], x.ptr, v["xx"][1].ptr,
+                                       1 if (l + 1) % 6 == 0 else 0, ws.ptr, st))
+        fr.check(lib.frhip_head(C_, x.ptr, ln_o[0].ptr, ln_o[1].ptr, C.byref(head), logits.ptr, st))
+
+    fr.check(lib.frhip_graph_begin(st))
+    token()
+    g = C.c_void_p()
+    fr.check(lib.frhip_graph_end(st, C.byref(g)))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.frhip_event_create(C.byref(e0))
+    lib.frhip_event_create(C.byref(e1))
+    for _ in range(3):
+        fr.check(lib.frhip_graph_launch(g, st))
+    fr.check(lib.frhip_stream_sync(st))
+    fr.check(lib.frhip_event_record(e0, st))
+    for _ in range(reps):
+        fr.check(lib.frhip_graph_launch(g, st))
+    fr.check(lib.frhip_event_record(e1, st))
+    fr.check(lib.frhip_event_sync(e1))
+    ms = C.c_float()
+    fr.check(lib.frhip_event_elapsed_ms(e0, e1, C.byref(ms)))
+    lib.frhip_graph_destroy(g)
+    lib.frhip_stream_destroy(st)
+    n_launch = 4 * L_ + 1
+    return ms.value / reps, n_launch
+
+
+def cpu_baseline(seconds_budget=20.0):
+    """The oracle's fp32 one-token forward on the host cores (OpenMP over output columns), on
+    the same architecture with the depth cut to 2 layers + head to bound the run; the
+    per-token time is scaled to 24 layers by the measured per-layer time."""
+    import pyoracle as po
+    rng = np.random.default_rng(1)
+    Ls = 2
+
+    def mat(k, n):
+        return (rng.standard_normal((k, n), dtype=np.float32) * 0.02)
+
+    def vec(lo, hi):
+        return rng.uniform(lo, hi, C_).astype(np.float32)
+
+    params = []
+    for _ in range(Ls):
+        params += [np.ones(C_, np.float32), np.zeros(C_, np.float32), vec(0, 1), vec(0, 1), vec(0, 1),
+                   -np.exp(vec(-5, 1)), vec(-1, 1), mat(C_, C_), mat(C_, C_), mat(C_, C_), mat(C_, C_),
+                   np.ones(C_, np.float32), np.zeros(C_, np.float32), vec(0, 1), vec(0, 1), mat(C_, F_), mat(F_, C_),
+                   mat(C_, C_)]
+    params += [np.ones(C_, np.float32), np.zeros(C_, np.float32), mat(C_, V_)]
+    emb = rng.standard_normal((1024, C_), dtype=np.float32)
+    full = po.Model(4, po.F32, Ls, C_, F_, 0, V_, params, emb)
+    shallow = po.Model(4, po.F32, 1, C_, F_, 0, V_, params[:18] + params[-3:], emb)
+
+    def per_token(m, budget):
+        m.run(1)
+        n, t0 = 0, time.perf_counter()
+        while True:
+            m.run(n % 1024)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt > budget or n >= 64:
+                return dt / n, n
+
+    t2, n2 = per_token(full, seconds_budget * 0.6)
+    t1, n1 = per_token(shallow, seconds_budget * 0.4)
+    per_layer = max(t2 - t1, 1e-9)
+    head_t = max(t1 - per_layer, 0.0)
+    t24 = L_ * per_layer + head_t
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(1.0 / t24, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "sample": "oracle fp32 one-token forward, 2-layer and 1-layer slices of the 1.5B shape + 65536 head, "
+                      "%d+%d tokens timed; per-layer time x24 + head" % (n2, n1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=512)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--dtype", choices=["fp16", "int8"], default="fp16")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs batch-1 decode on ONE GPU; --gpus %d is not supported "
+                 "(no multi-GPU path exists or is measured)" % args.gpus)
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: launched with WORLD_SIZE > 1; only a single rank is supported")
+
+    fr = importlib.import_module("faster-rwkv_amd")
+    cfg = CONFIGS[args.dtype]
+    t0 = time.perf_counter()
+    model = fr.Model(cfg["spec"], cfg["strategy"])
+    build_s = time.perf_counter() - t0
+    print("[bench] model built in %.1f s: %s" % (build_s, cfg["workload"]), file=sys.stderr, flush=True)
+
+    model.greedy(0, args.warmup)
+    fr.check(fr.lib().frhip_device_sync())
+    toks, secs = model.greedy(17, args.steps)
+    fr.check(fr.lib().frhip_device_sync())
+    model.close()
+    ms_per_step = 1e3 * secs / args.steps
+    tok_s = args.steps / secs
+
+    kernel_ms, n_launch = measure_kernels(fr, cfg)
+    abytes = algorithmic_bytes_per_token(cfg["wbytes"])
+    achieved = abytes / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "decode tok/s (RWKV-4 1.5B-shaped, bs1, greedy)", "value": round(tok_s, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if args.dtype == "fp16" else "u8 weights, f16 activations, f32 accumulate",
+        "data": "synthetic (random-init weights, greedy token ids)",
+        "config": {"workload": cfg["workload"], "strategy": cfg["strategy"], "steps": args.steps,
+                   "host_loop": "Model::Run + D2H logits + host argmax per token"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "row-streaming matrix-vector kernels (att_front/att_out/ffn_front/ffn_out/head), "
+                               "%d launches per token" % n_launch,
+                     "bytes_per_token": abytes, "kernel_ms_per_token": round(kernel_ms, 4),
+                     "avg_launch_us": round(1e3 * kernel_ms / n_launch, 3)},
+        "roofline_tok_s": round(1.0 / (abytes / (HBM_PEAK_GBS * 1e9)), 1),
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

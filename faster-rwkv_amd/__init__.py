@@ -81,6 +81,7 @@ _SIGS = {
     "frhip_fill": (_i, [_vp, _i, C.c_float, _sz, _vp]),
     "frhip_scalar_div_f16": (_i, [_vp, C.c_float, _sz, _vp]),
     "frhip_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "frhip_embed_ring": (_i, [_vp, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "frhip_decode_workspace_bytes": (_sz, [_i, _i]),
     "frhip_att_one_v4": (_i, [_i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),
     "frhip_ffn_one": (_i, [_i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
@@ -208,3 +209,138 @@ class PackedWeight:
     @property
     def ref(self):
         return C.byref(self.c)
+
+
+# --------------------------------------------------------------------------
+# host layer (libfr_host.so): rwkv::Model through its C API
+# --------------------------------------------------------------------------
+_host = None
+
+
+def host():
+    global _host
+    if _host is None:
+        if not os.path.exists(LIBHOST):
+            raise FrhipError("libfr_host.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
+        lib()  # libfrhip.so first, so that the dependency resolves to the in-tree copy
+        h = C.CDLL(LIBHOST)
+        h.fr_last_error.restype = C.c_char_p
+        h.fr_model_create.restype = _vp
+        h.fr_model_create.argtypes = [C.c_char_p, C.c_char_p]
+        h.fr_model_free.argtypes = [_vp]
+        h.fr_model_info.argtypes = [_vp, C.POINTER(_i)]
+        h.fr_model_run.argtypes = [_vp, _vp, _i, _vp, _i]
+        h.fr_model_reset.argtypes = [_vp]
+        h.fr_model_save_state.argtypes = [_vp, C.c_char_p]
+        h.fr_model_load_state.argtypes = [_vp, C.c_char_p]
+        h.fr_model_get_state.argtypes = [_vp, _i, _i, _vp, _i]
+        h.fr_greedy_decode.restype = C.c_longlong
+        h.fr_greedy_decode.argtypes = [_vp, _i, _i, _vp]
+        h.fr_quantize_u8.argtypes = [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp]
+        h.fr_allocator_stats.argtypes = [C.POINTER(_sz)] * 3
+        _host = h
+    return _host
+
+
+class Model:
+    """rwkv::Model(path, strategy) -- strategy "hip fp16" or "hip int8"; path a .fr file or
+    "synthetic:v=4,L=..,C=..,F=..,V=..,seed=.."."""
+
+    def __init__(self, path, strategy):
+        self._h = host()
+        self._m = self._h.fr_model_create(path.encode(), strategy.encode())
+        if not self._m:
+            raise FrhipError("Model(%r, %r): %s" % (path, strategy, self._h.fr_last_error().decode()))
+        info = (_i * 6)()
+        self._chk(self._h.fr_model_info(self._m, info))
+        self.n_layer, self.n_embd, self.n_att, self.n_ffn, self.n_head, self.vocab = list(info)
+        self._logits = np.empty(1 << 20, np.float32)
+
+    def _chk(self, rc):
+        if rc < 0:
+            raise FrhipError(self._h.fr_last_error().decode())
+        return rc
+
+    def run(self, ids):
+        """Model::Run: an int runs one token, a sequence runs seq mode; returns fp32 logits."""
+        ids = np.atleast_1d(np.asarray(ids, np.int32))
+        n = self._chk(self._h.fr_model_run(self._m, ids.ctypes.data, len(ids), self._logits.ctypes.data,
+                                           self._logits.size))
+        return self._logits[:n].copy()
+
+    def reset(self):
+        self._chk(self._h.fr_model_reset(self._m))
+
+    def save_state(self, path):
+        self._chk(self._h.fr_model_save_state(self._m, path.encode()))
+
+    def load_state(self, path):
+        self._chk(self._h.fr_model_load_state(self._m, path.encode()))
+
+    def state(self, layer, index, dtype):
+        buf = np.empty(1 << 22, np.uint8)
+        n = self._chk(self._h.fr_model_get_state(self._m, layer, index, buf.ctypes.data, buf.size))
+        return buf[:n].view(dtype).copy()
+
+    def greedy(self, first_id, steps):
+        """chat.cpp's greedy loop in C++; returns (token ids, seconds)."""
+        out = np.empty(steps, np.int32)
+        us = self._h.fr_greedy_decode(self._m, int(first_id), int(steps), out.ctypes.data)
+        if us < 0:
+            raise FrhipError(self._h.fr_last_error().decode())
+        return out, us * 1e-6
+
+    def close(self):
+        if getattr(self, "_m", None):
+            self._h.fr_model_free(self._m)
+            self._m = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def write_fr(path, version, n_layer, n_embd, n_ffn, n_head, params, emb, quantized=None):
+    """Write a `.fr` file (msgpack layout of tools/convert_weight.py:12-55) from numpy arrays in
+    the positional parameter order.  `quantized` maps a parameter index to (q, mx, rx, my, ry)."""
+    import msgpack
+    names = []
+    for l in range(n_layer):
+        b, a, f = "blocks.%d." % l, "blocks.%d.att." % l, "blocks.%d.ffn." % l
+        names += [b + "ln1.weight", b + "ln1.bias"]
+        if version != "4":
+            names += [a + "ln_x.weight", a + "ln_x.bias"]
+        names += [a + "time_mix_k", a + "time_mix_v", a + "time_mix_r"]
+        if version in ("5.1", "5.2"):
+            names += [a + "time_mix_g"]
+        names += [a + "time_decay", a + "time_first", a + "key.weight", a + "value.weight", a + "receptance.weight"]
+        if version in ("5.1", "5.2"):
+            names += [a + "gate.weight"]
+        names += [a + "output.weight", b + "ln2.weight", b + "ln2.bias", f + "time_mix_k", f + "time_mix_r",
+                  f + "key.weight", f + "value.weight", f + "receptance.weight"]
+    names += ["ln_out.weight", "ln_out.bias", "head.weight"]
+    assert len(names) == len(params), (len(names), len(params))
+    tname = {np.dtype(np.float16): "torch.float16", np.dtype(np.float32): "torch.float32",
+             np.dtype(np.uint8): "torch.uint8"}
+
+    def pack(a):
+        a = np.ascontiguousarray(a)
+        return {"dtype": tname[a.dtype], "data": a.tobytes(), "shape": list(a.shape)}
+
+    weights = {}
+    for i, (n, p) in enumerate(zip(names, params)):
+        if quantized and i in quantized:
+            q, mx, rx, my, ry = quantized[i]
+            weights[n] = pack(q)
+            for suf, v in (("_mx", mx), ("_rx", rx), ("_my", my), ("_ry", ry)):
+                weights[n + suf] = pack(np.asarray(v, np.float16))
+        else:
+            weights[n] = pack(p)
+    d = {"embd_weights": [pack(r) for r in emb], "weights": weights, "version": version, "n_layer": n_layer,
+         "n_embd": n_embd, "n_att": n_embd, "n_ffn": n_ffn}
+    if version != "4":
+        d["n_head"] = n_head
+    with open(path, "wb") as fh:
+        msgpack.pack(d, fh, use_bin_type=True)

@@ -89,6 +89,23 @@ __global__ void gather_rows_kernel(const unsigned char* __restrict__ table, cons
   for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x) dst[i] = src[i];
 }
 
+__global__ __launch_bounds__(256) void embed_ring_kernel(const unsigned char* __restrict__ table, int n_rows,
+                                                         int row_bytes, const int32_t* ring, int ring_len,
+                                                         uint32_t* counter, unsigned char* __restrict__ out) {
+  __shared__ int row;
+  if (threadIdx.x == 0) {
+    const uint32_t c = *counter;
+    int id = ring[c % (uint32_t)ring_len];
+    id = id < 0 ? 0 : (id >= n_rows ? n_rows - 1 : id);
+    row = id;
+    *counter = c + 1;
+  }
+  __syncthreads();
+  const u32x4* src = reinterpret_cast<const u32x4*>(table + (size_t)row * row_bytes);
+  u32x4* dst = reinterpret_cast<u32x4*>(out);
+  for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x) dst[i] = src[i];
+}
+
 // [K][N] -> [N][K] through a 64x64 LDS tile (+1 padding against bank conflicts).
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst, int K, int N) {
@@ -244,6 +261,16 @@ int frhip_gather_rows(const void* table, const int32_t* ids_dev, void* out, int 
   hipLaunchKernelGGL(gather_rows_kernel, dim3(n_ids), dim3(256), 0, static_cast<hipStream_t>(s),
                      (const unsigned char*)table, ids_dev, (unsigned char*)out, row_bytes);
   return check_launch("gather_rows");
+}
+
+int frhip_embed_ring(const void* table, int n_rows, int row_bytes, const int32_t* ring, int ring_len,
+                     uint32_t* counter_dev, void* out, frhip_stream s) {
+  if (!table || !ring || !counter_dev || !out) return set_error(FRHIP_EINVAL, "embed_ring: null pointer");
+  if (n_rows <= 0 || ring_len <= 0 || row_bytes <= 0 || row_bytes % 16 != 0)
+    return set_error(FRHIP_ESHAPE, "embed_ring: row_bytes must be a positive multiple of 16");
+  hipLaunchKernelGGL(embed_ring_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(s),
+                     (const unsigned char*)table, n_rows, row_bytes, ring, ring_len, counter_dev, (unsigned char*)out);
+  return check_launch("embed_ring");
 }
 
 int frhip_pack_transpose(const void* src, void* dst, int K, int N, int elem_bytes, frhip_stream s) {

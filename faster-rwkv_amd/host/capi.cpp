@@ -1,0 +1,154 @@
+// A small C API over rwkv::Model for scripts and benchmarks (ctypes).  It adds nothing to
+// the model; it only lets a non-C++ caller construct a Model with a strategy string, run
+// it, and read the logits -- what chat.cpp / bench_model.cpp do in the reference.
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <string>
+
+#include "kernels/hip/context.h"
+#include "kernels/kernels.h"
+#include "model.h"
+
+namespace rwkv::hip {
+void allocator_stats(size_t *reserved, size_t *in_use, size_t *driver_calls);
+}
+
+namespace {
+thread_local std::string g_err;
+template <typename F> int guarded(F &&f) {
+  try {
+    return f();
+  } catch (const std::exception &e) {
+    g_err = e.what();
+    return -1;
+  }
+}
+// First index of the maximum (Sampler::Sample with top_k = 1).  Two passes so that the
+// compiler can vectorise the first: eight independent running maxima, then a scan for the value.
+int argmax(const float *x, int n) {
+  float m[8];
+  for (int j = 0; j < 8; j++) m[j] = -INFINITY;
+  int i = 0;
+  for (; i + 8 <= n; i += 8)
+    for (int j = 0; j < 8; j++) m[j] = x[i + j] > m[j] ? x[i + j] : m[j];
+  float best = m[0];
+  for (int j = 1; j < 8; j++) best = m[j] > best ? m[j] : best;
+  for (; i < n; i++) best = x[i] > best ? x[i] : best;
+  for (i = 0; i < n; i++)
+    if (x[i] == best) return i;
+  return 0;
+}
+}  // namespace
+
+extern "C" {
+
+const char *fr_last_error(void) { return g_err.c_str(); }
+
+void *fr_model_create(const char *path, const char *strategy) {
+  void *m = nullptr;
+  guarded([&]() {
+    m = new rwkv::Model(path, strategy);
+    return 0;
+  });
+  return m;
+}
+
+void fr_model_free(void *m) { delete static_cast<rwkv::Model *>(m); }
+
+// out[0..5] = n_layer, n_embd, n_att, n_ffn, n_head, vocab
+int fr_model_info(void *m, int *out) {
+  return guarded([&]() {
+    auto *model = static_cast<rwkv::Model *>(m);
+    out[0] = model->n_layer();
+    out[1] = model->n_embd();
+    out[2] = model->n_att();
+    out[3] = model->n_ffn();
+    out[4] = model->head_size();
+    out[5] = static_cast<int>(model->_embd_weights.size());
+    return 0;
+  });
+}
+
+// Model::Run(ids): n == 1 one-token forward, n > 1 seq mode.  Returns the number of logits.
+int fr_model_run(void *m, const int *ids, int n, float *logits, int capacity) {
+  return guarded([&]() {
+    auto *model = static_cast<rwkv::Model *>(m);
+    rwkv::Tensor out = n == 1 ? model->Run(ids[0]) : model->Run(std::vector<int>(ids, ids + n));
+    const int v = static_cast<int>(out.numel());
+    if (v > capacity) throw FRException("logits buffer too small");
+    std::memcpy(logits, out.data_ptr<float>(), sizeof(float) * static_cast<size_t>(v));
+    return v;
+  });
+}
+
+int fr_model_reset(void *m) {
+  return guarded([&]() {
+    static_cast<rwkv::Model *>(m)->ResetStates();
+    return 0;
+  });
+}
+
+int fr_model_save_state(void *m, const char *path) {
+  return guarded([&]() {
+    static_cast<rwkv::Model *>(m)->SaveStateFile(path);
+    return 0;
+  });
+}
+
+int fr_model_load_state(void *m, const char *path) {
+  return guarded([&]() {
+    static_cast<rwkv::Model *>(m)->LoadStateFile(path);
+    return 0;
+  });
+}
+
+// Copy state tensor (layer, index) to the host as raw bytes; returns its size in bytes.
+int fr_model_get_state(void *m, int layer, int index, void *out, int capacity) {
+  return guarded([&]() {
+    auto *model = static_cast<rwkv::Model *>(m);
+    rwkv::Tensor c = rwkv::Copy(model->states().at(layer).at(index), rwkv::Device::kCPU);
+    const int n = static_cast<int>(c.nbytes());
+    if (n > capacity) throw FRException("state buffer too small");
+    std::memcpy(out, c.data_ptr(), static_cast<size_t>(n));
+    return n;
+  });
+}
+
+// Greedy decoding as chat.cpp:56-92 does with top_k = 1: feed `first_id`, take the argmax of
+// the returned (host) logits, feed it back.  out_ids receives `steps` tokens.  Returns the
+// wall time of the loop in microseconds (>= 0) or -1.
+long long fr_greedy_decode(void *m, int first_id, int steps, int *out_ids) {
+  long long us = -1;
+  guarded([&]() {
+    auto *model = static_cast<rwkv::Model *>(m);
+    int id = first_id;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; i++) {
+      rwkv::Tensor out = model->Run(id);
+      id = argmax(out.data_ptr<float>(), static_cast<int>(out.numel()));
+      out_ids[i] = id;
+    }
+    const auto t1 = std::chrono::steady_clock::now();
+    us = std::chrono::duration_cast<std::chrono::microseconds>(t1 - t0).count();
+    return 0;
+  });
+  return us;
+}
+
+int fr_quantize_u8(const uint16_t *w_kn, int K, int N, uint8_t *q, uint16_t *mx, uint16_t *rx, uint16_t *my,
+                   uint16_t *ry) {
+  return guarded([&]() {
+    rwkv::hip::quantize_u8(w_kn, K, N, q, mx, rx, my, ry);
+    return 0;
+  });
+}
+
+int fr_allocator_stats(size_t *reserved, size_t *in_use, size_t *driver_calls) {
+  return guarded([&]() {
+    rwkv::hip::allocator_stats(reserved, in_use, driver_calls);
+    return 0;
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,195 @@
+// model_forward / model_forward_seq for Device::kHIP.
+//
+// One token of RWKV-4 is 4 fused launches per layer plus gather and head (98 for a
+// 24-layer model, against ~415 in kernels/default/model_forward.cpp:105-188 over
+// kernels/cuda).  All buffers are fixed for the life of the model, so the whole token is
+// captured once into a HIP graph and replayed.  The token-shift states ping-pong between
+// two buffers (the kernel that writes the new state runs while other workgroups still read
+// the old one), hence one graph per parity.  The token id reaches the first kernel through a
+// small ring in pinned host memory, and the graph's last node copies the logits to pinned host
+// memory, so a step costs the host one graph launch and one stream wait.  The recurrent state that model code sees
+// (Model::states()) is kept as views of these buffers; states assigned from outside
+// (ResetStates, LoadStateFile, set_states) are copied in on the next call.
+//
+// FR_HIP_GENERIC=1 selects the operator-by-operator loop instead; FR_HIP_NO_GRAPH=1 keeps
+// the fused path but launches eagerly.
+#include <cstdlib>
+
+#include "kernels/hip/context.h"
+#include "kernels/hip/hip_model.h"
+#include "kernels/kernels.h"
+#include "kernels/registry.h"
+#include "model.h"
+
+namespace rwkv {
+namespace hip {
+
+struct DecodePlan {
+  static constexpr int kRing = 64;
+  int L = 0, C = 0, F = 0, V = 0, n_logits = 0;
+  Tensor x, ws, counter;
+  Tensor logits_dev;
+  float *logits_host[2] = {nullptr, nullptr};  // pinned; the graph's last node copies into it
+  int32_t *ring = nullptr;                     // pinned; token ids, read by the first kernel
+  uint32_t fed = 0;                            // tokens fed so far == the device counter
+  std::vector<Tensor> aa, bb, pp;
+  std::vector<Tensor> sx_att[2], sx_ffn[2];
+  std::vector<std::vector<Tensor>> views[2];  // views[parity][layer] = the 5 state tensors model code sees
+  int parity = 0;                             // which ping-pong side holds the current shift states
+  frhip_graph graph[2] = {nullptr, nullptr};
+  bool use_graph = true;
+  ~DecodePlan() {
+    for (auto g : graph)
+      if (g) frhip_graph_destroy(g);
+    if (ring) frhip_host_free(ring);
+    for (auto h : logits_host)
+      if (h) frhip_host_free(h);
+  }
+};
+
+static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
+  auto p = std::make_shared<DecodePlan>();
+  p->L = model->n_layer();
+  p->C = model->n_embd();
+  p->F = model->n_ffn() > 0 ? model->n_ffn() : static_cast<int>(model->_params[15].size(1));
+  p->V = static_cast<int>(ex.emb_table.size(0));
+  const int C = p->C;
+  const Device d = Device::kHIP;
+  p->x = Tensor::Empty({C}, DType::kFloat16, d);
+  p->ws = Tensor::Empty({static_cast<LengthType>(frhip_decode_workspace_bytes(C, p->F))}, DType::kInt8, d);
+  p->counter = Tensor::Empty({1}, DType::kInt32, d);
+  FRHIP_CHECK(frhip_fill(p->counter.data_ptr(), FRHIP_F32, 0.0f, 1, stream()));  // all-zero bits
+  p->n_logits = static_cast<int>(model->_params.back().size(1));
+  p->logits_dev = Tensor::Empty({p->n_logits}, DType::kFloat32, d);
+  void *h = nullptr;
+  FRHIP_CHECK(frhip_host_malloc(&h, sizeof(int32_t) * DecodePlan::kRing));
+  p->ring = static_cast<int32_t *>(h);
+  for (auto &lh : p->logits_host) {
+    FRHIP_CHECK(frhip_host_malloc(&h, sizeof(float) * static_cast<size_t>(p->n_logits)));
+    lh = static_cast<float *>(h);
+  }
+  for (int l = 0; l < p->L; l++) {
+    p->aa.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+    p->bb.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+    p->pp.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+    for (int s = 0; s < 2; s++) {
+      p->sx_att[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
+      p->sx_ffn[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
+    }
+  }
+  for (int s = 0; s < 2; s++) {
+    p->views[s].resize(p->L);
+    for (int l = 0; l < p->L; l++)
+      p->views[s][l] = {p->sx_att[s][l], p->aa[l], p->bb[l], p->pp[l], p->sx_ffn[s][l]};
+  }
+  p->use_graph = std::getenv("FR_HIP_NO_GRAPH") == nullptr;  // fixed when the model first runs
+  return p;
+}
+
+// Bring states assigned from outside into the plan's buffers and rebind the model's
+// state tensors to them.
+static void adopt_states(Model *model, DecodePlan &p) {
+  auto &st = model->states();
+  RV_CHECK(static_cast<int>(st.size()) == p.L);
+  for (int l = 0; l < p.L; l++) {
+    RV_CHECK(st[l].size() == 5);
+    auto &mine = p.views[p.parity][l];
+    for (int j = 0; j < 5; j++) {
+      if (st[l][j].data_ptr() == mine[j].data_ptr()) continue;
+      RV_CHECK(st[l][j].nbytes() == mine[j].nbytes() && st[l][j].dtype() == mine[j].dtype())
+          << "state " << l << "/" << j << " has the wrong shape or dtype";
+      Tensor src = st[l][j].device() == Device::kHIP ? st[l][j] : Copy(st[l][j], Device::kHIP);
+      FRHIP_CHECK(frhip_memcpy_async(mine[j].data_ptr(), src.data_ptr(), src.nbytes(), FRHIP_D2D, stream()));
+      if (src.data_ptr() != st[l][j].data_ptr()) FRHIP_CHECK(frhip_stream_sync(stream()));  // src dies here
+      st[l][j] = mine[j];
+    }
+  }
+}
+
+static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
+  const auto &P = model->_params;
+  frhip_stream s = stream();
+  const int C = p.C, F = p.F;
+  const int cur = p.parity, nxt = 1 - p.parity;
+  FRHIP_CHECK(frhip_embed_ring(ex.emb_table.data_ptr(), p.V, 2 * C, p.ring, DecodePlan::kRing,
+                               reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
+  size_t pi = 0;
+  for (int l = 0; l < p.L; l++) {
+    const frhip_weight *kw = find_weight(P[pi + 7]), *vw = find_weight(P[pi + 8]), *rw = find_weight(P[pi + 9]),
+                       *ow = find_weight(P[pi + 10]);
+    RV_CHECK(kw && vw && rw && ow);
+    FRHIP_CHECK(frhip_att_one_v4(C, p.x.data_ptr(), p.sx_att[cur][l].data_ptr(), p.aa[l].data_ptr<float>(),
+                                 p.bb[l].data_ptr<float>(), p.pp[l].data_ptr<float>(), P[pi].data_ptr(),
+                                 P[pi + 1].data_ptr(), P[pi + 2].data_ptr(), P[pi + 3].data_ptr(),
+                                 P[pi + 4].data_ptr(), P[pi + 5].data_ptr<float>(), P[pi + 6].data_ptr<float>(), kw,
+                                 vw, rw, ow, p.x.data_ptr(), p.sx_att[nxt][l].data_ptr(), p.aa[l].data_ptr<float>(),
+                                 p.bb[l].data_ptr<float>(), p.pp[l].data_ptr<float>(), p.ws.data_ptr(), s));
+    pi += 11;
+    const frhip_weight *fk = find_weight(P[pi + 4]), *fv = find_weight(P[pi + 5]), *frw = find_weight(P[pi + 6]);
+    RV_CHECK(fk && fv && frw);
+    FRHIP_CHECK(frhip_ffn_one(C, F, p.x.data_ptr(), p.sx_ffn[cur][l].data_ptr(), P[pi].data_ptr(),
+                              P[pi + 1].data_ptr(), P[pi + 2].data_ptr(), P[pi + 3].data_ptr(), fk, fv, frw,
+                              p.x.data_ptr(), p.sx_ffn[nxt][l].data_ptr(), (l + 1) % 6 == 0 ? 1 : 0, p.ws.data_ptr(),
+                              s));
+    pi += 7;
+  }
+  const frhip_weight *hw = find_weight(P[pi + 2]);
+  RV_CHECK(hw != nullptr);
+  FRHIP_CHECK(frhip_head(C, p.x.data_ptr(), P[pi].data_ptr(), P[pi + 1].data_ptr(), hw,
+                         p.logits_dev.data_ptr<float>(), s));
+  FRHIP_CHECK(frhip_memcpy_async(p.logits_host[cur], p.logits_dev.data_ptr(), sizeof(float) * (size_t)p.n_logits,
+                                 FRHIP_D2H, s));
+}
+
+Tensor ModelForward(Model *model, Device device, int id) {
+  const bool generic = std::getenv("FR_HIP_GENERIC") != nullptr;  // read per call so that one process can compare both paths
+  if (generic || model->version() != "4") return def::ModelForward(model, device, id);
+  auto ex = extra_of(model);
+  if (!ex->plan) ex->plan = make_plan(model, *ex);
+  DecodePlan &p = *ex->plan;
+  RV_CHECK(id >= 0 && id < p.V) << "token id " << id << " out of range";
+  adopt_states(model, p);
+  frhip_stream s = stream();
+  // every call ends with a stream synchronisation, so the device has consumed all earlier slots
+  p.ring[p.fed % DecodePlan::kRing] = id;
+  const int cur = p.parity;
+  if (!p.use_graph) {
+    issue_token(model, *ex, p);
+  } else {
+    if (!p.graph[cur]) {
+      FRHIP_CHECK(frhip_graph_begin(s));
+      try {
+        issue_token(model, *ex, p);
+      } catch (...) {
+        frhip_graph g = nullptr;
+        frhip_graph_end(s, &g);
+        if (g) frhip_graph_destroy(g);
+        throw;
+      }
+      FRHIP_CHECK(frhip_graph_end(s, &p.graph[cur]));
+    }
+    FRHIP_CHECK(frhip_graph_launch(p.graph[cur], s));
+  }
+  p.fed++;  // the device counter advances when the first kernel of the step runs
+  p.parity = 1 - cur;
+  auto &st = model->states();
+  for (int l = 0; l < p.L; l++) {
+    st[l][0] = p.views[p.parity][l][0];
+    st[l][4] = p.views[p.parity][l][4];
+  }
+  // The graph's last node has copied the logits into pinned host memory; waiting for the stream
+  // is the step's one synchronisation point (the reference's is the blocking cudaMemcpy in
+  // tensor.cpp:65-68).  The returned CPU tensor is a view, valid until the next-but-one call.
+  FRHIP_CHECK(frhip_stream_sync(s));
+  return Tensor::FromPtr(p.logits_host[cur], {p.n_logits}, DType::kFloat32, Device::kCPU);
+}
+
+Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids, bool full_output) {
+  return def::ModelForwardSeqFallback(model, device, ids, full_output);
+}
+
+KernelRegister model_forward_reg("model_forward", Device::kHIP, ModelForward);
+KernelRegister model_forward_seq_reg("model_forward_seq", Device::kHIP, ModelForwardSeq);
+
+}  // namespace hip
+}  // namespace rwkv

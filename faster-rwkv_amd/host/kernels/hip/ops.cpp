@@ -1,0 +1,175 @@
+// Operators registered for Device::kHIP.  Each is a thin host function: it checks
+// shapes, allocates outputs through the device allocator, and calls the C ABI of
+// libfrhip.so with raw pointers.  Signatures are the ones kernels/kernels.h dispatches to.
+#include <cstring>
+
+#include "kernels/hip/context.h"
+#include "kernels/kernels.h"
+#include "kernels/registry.h"
+
+namespace rwkv {
+namespace hip {
+
+namespace {
+
+int to_frhip_dtype(DType d) {
+  if (d == DType::kFloat16) return FRHIP_F16;
+  if (d == DType::kFloat32) return FRHIP_F32;
+  if (d == DType::kInt8) return FRHIP_U8;
+  RV_UNIMPLEMENTED() << "dtype " << dtype_to_string(d) << " on hip";
+}
+
+// Packed description of a weight tensor.  A tensor that did not come from init_model
+// (a plain [K, N] binary16 matrix on the device) is packed on the fly into `tmp`.
+const frhip_weight *weight_of(const Tensor &w, frhip_weight &tmp_desc, Tensor &tmp) {
+  if (const frhip_weight *p = find_weight(w)) return p;
+  RV_CHECK(w.shape().size() == 2 && w.dtype() == DType::kFloat16)
+      << "matmul on hip: right operand must be a packed weight or a 2-D fp16 tensor";
+  const int K = static_cast<int>(w.size(0)), N = static_cast<int>(w.size(1));
+  tmp = Tensor::Empty({N, K}, DType::kFloat16, Device::kHIP);
+  FRHIP_CHECK(frhip_pack_transpose(w.data_ptr(), tmp.data_ptr(), K, N, 2, stream()));
+  std::memset(&tmp_desc, 0, sizeof(tmp_desc));
+  tmp_desc.data = tmp.data_ptr();
+  tmp_desc.K = K;
+  tmp_desc.N = N;
+  tmp_desc.dtype = FRHIP_F16;
+  return &tmp_desc;
+}
+
+Tensor workspace(int C, int F) {
+  const size_t bytes = frhip_decode_workspace_bytes(C, F);
+  return Tensor::Empty({static_cast<LengthType>(bytes)}, DType::kInt8, Device::kHIP);
+}
+
+}  // namespace
+
+Tensor &fill_(Tensor &x, float value) {
+  FRHIP_CHECK(frhip_fill(x.data_ptr(), to_frhip_dtype(x.dtype()), value, static_cast<size_t>(x.numel()), stream()));
+  return x;
+}
+
+Tensor cast_dtype(const Tensor &x, DType dtype) {
+  if (x.dtype() == dtype) return x;
+  Tensor y = Tensor::Empty(x.shape(), dtype, Device::kHIP);
+  FRHIP_CHECK(frhip_cast(x.data_ptr(), to_frhip_dtype(x.dtype()), y.data_ptr(), to_frhip_dtype(dtype),
+                         static_cast<size_t>(x.numel()), stream()));
+  return y;
+}
+
+Tensor scalar_div_(Tensor &x, float value) {
+  RV_CHECK(x.dtype() == DType::kFloat16) << "scalar_div_ on hip is defined for fp16 (model_forward.cpp:173-175)";
+  FRHIP_CHECK(frhip_scalar_div_f16(x.data_ptr(), value, static_cast<size_t>(x.numel()), stream()));
+  return x;
+}
+
+Tensor layernorm(const Tensor &x, const Tensor &weight, const Tensor &bias) {
+  RV_CHECK(x.sizes().size() <= 2);
+  RV_CHECK(x.dtype() == weight.dtype() && x.dtype() == bias.dtype());
+  const int rows = x.sizes().size() == 1 ? 1 : static_cast<int>(x.size(0));
+  const int cols = static_cast<int>(x.size(-1));
+  Tensor y = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_layernorm(x.data_ptr(), weight.data_ptr(), bias.data_ptr(), y.data_ptr(), rows, cols,
+                              to_frhip_dtype(x.dtype()), stream()));
+  return y;
+}
+
+Tensor groupnorm(const Tensor &x, int num_groups, const Tensor &weight, const Tensor &bias) {
+  RV_CHECK(x.sizes().size() <= 2);
+  RV_CHECK(x.dtype() == DType::kFloat32 && weight.dtype() == DType::kFloat32 && bias.dtype() == DType::kFloat32)
+      << "groupnorm on hip runs on fp32 (the dtype the RWKV-5 path gives it)";
+  const int rows = x.sizes().size() == 1 ? 1 : static_cast<int>(x.size(0));
+  const int cols = static_cast<int>(x.size(-1));
+  Tensor y = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_groupnorm_f32(x.data_ptr<float>(), num_groups, weight.data_ptr<float>(), bias.data_ptr<float>(),
+                                  y.data_ptr<float>(), rows, cols, stream()));
+  return y;
+}
+
+// matmul (reference: kernels/cuda/matmul.cpp:123-146).  Vector x matrix runs the
+// row-streaming kernel; output dtype = activation dtype.
+Tensor matmul(const Tensor &a, const Tensor &b) {
+  RV_CHECK(a.device() == b.device());
+  RV_CHECK(a.dtype() == DType::kFloat16) << "matmul on hip: activations are fp16";
+  RV_CHECK(a.sizes().size() == 1 && b.sizes().size() == 2) << "matmul on hip: vector x matrix only on this path";
+  RV_CHECK(a.size(0) == b.size(0)) << "matmul: " << shape_str(a.shape()) << " x " << shape_str(b.shape());
+  frhip_weight tmp_desc;
+  Tensor tmp;
+  const frhip_weight *w = weight_of(b, tmp_desc, tmp);
+  Tensor c = Tensor::Empty({b.size(1)}, a.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_gemv(a.data_ptr(), w, c.data_ptr(), FRHIP_F16, stream()));
+  return c;
+}
+
+// vgather (reference: kernels/default/gather_ops.cpp:46-89): rows are copied device to
+// device.  When the rows are views into one table (as this backend's init_model makes
+// them) the copies are contiguous slices of that table.
+Tensor vgather(const std::vector<Tensor> &x, const std::vector<int> &idx) {
+  Shape shape{static_cast<LengthType>(idx.size())};
+  shape.insert(shape.end(), x[0].shape().begin(), x[0].shape().end());
+  Tensor out = Tensor::Empty(shape, x[0].dtype(), Device::kHIP);
+  const size_t row = x[0].nbytes();
+  char *dst = static_cast<char *>(out.data_ptr());
+  for (size_t i = 0; i < idx.size(); i++) {
+    RV_CHECK(idx[i] >= 0 && static_cast<size_t>(idx[i]) < x.size());
+    FRHIP_CHECK(frhip_memcpy_async(dst + i * row, x[idx[i]].data_ptr(), row, FRHIP_D2D, stream()));
+  }
+  return out;
+}
+
+// att, RWKV-4 one token (reference: kernels/cuda/att.cu:337-359).
+std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor>
+att(const Tensor &x, const Tensor &sx, const Tensor &aa, const Tensor &bb, const Tensor &pp, const Tensor &ln_w,
+    const Tensor &ln_b, const Tensor &k_mix, const Tensor &v_mix, const Tensor &r_mix, const Tensor &t_decay,
+    const Tensor &t_first, const Tensor &kw, const Tensor &vw, const Tensor &rw, const Tensor &ow) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 1);
+  const int C = static_cast<int>(x.size(0));
+  frhip_weight d[4];
+  Tensor tmp[4];
+  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
+                              weight_of(ow, d[3], tmp[3])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor t1 = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor t2 = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor p = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor ws = workspace(C, 16);
+  FRHIP_CHECK(frhip_att_one_v4(C, x.data_ptr(), sx.data_ptr(), aa.data_ptr<float>(), bb.data_ptr<float>(),
+                               pp.data_ptr<float>(), ln_w.data_ptr(), ln_b.data_ptr(), k_mix.data_ptr(),
+                               v_mix.data_ptr(), r_mix.data_ptr(), t_decay.data_ptr<float>(),
+                               t_first.data_ptr<float>(), w[0], w[1], w[2], w[3], x_out.data_ptr(), xx.data_ptr(),
+                               t1.data_ptr<float>(), t2.data_ptr<float>(), p.data_ptr<float>(), ws.data_ptr(),
+                               stream()));
+  return {x_out, xx, t1, t2, p};
+}
+
+// ffn, one token (reference: kernels/cuda/ffn.cu:89-110).
+std::tuple<Tensor, Tensor> ffn(const Tensor &x, const Tensor &sx, const Tensor &ln_w, const Tensor &ln_b,
+                               const Tensor &k_mix, const Tensor &r_mix, const Tensor &kw, const Tensor &vw,
+                               const Tensor &rw) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 1);
+  const int C = static_cast<int>(x.size(0));
+  const int F = static_cast<int>(kw.size(1));
+  frhip_weight d[3];
+  Tensor tmp[3];
+  const frhip_weight *w[3] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor ws = workspace(C, F);
+  FRHIP_CHECK(frhip_ffn_one(C, F, x.data_ptr(), sx.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), k_mix.data_ptr(),
+                            r_mix.data_ptr(), w[0], w[1], w[2], x_out.data_ptr(), xx.data_ptr(), 0, ws.data_ptr(),
+                            stream()));
+  return {x_out, xx};
+}
+
+KernelRegister fill_reg("fill_", Device::kHIP, fill_);
+KernelRegister cast_reg("cast_dtype", Device::kHIP, cast_dtype);
+KernelRegister scalar_div_reg("scalar_div_", Device::kHIP, scalar_div_);
+KernelRegister layernorm_reg("layernorm", Device::kHIP, layernorm);
+KernelRegister groupnorm_reg("groupnorm", Device::kHIP, groupnorm);
+KernelRegister matmul_reg("matmul", Device::kHIP, matmul);
+KernelRegister vgather_reg("vgather", Device::kHIP, vgather);
+KernelRegister att_reg("att", Device::kHIP, att);
+KernelRegister ffn_reg("ffn", Device::kHIP, ffn);
+
+}  // namespace hip
+}  // namespace rwkv

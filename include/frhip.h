@@ -114,6 +114,14 @@ int frhip_scalar_div_f16(void *x, float divisor, size_t n, frhip_stream s);
 /* vgather of embedding rows: kernels/default/gather_ops.cpp:46-89.  table [V][C]; ids on the device. */
 int frhip_gather_rows(const void *table, const int32_t *ids_dev, void *out, int n_ids, int row_bytes, frhip_stream s);
 
+/* Token feed for a replayed graph: reads ring[*counter % ring_len] (ring may be pinned host
+ * memory, written by the host before the launch), advances *counter on the device, and copies
+ * that row of `table` to `out`.  Ids outside [0, n_rows) are clamped.  Replaces the per-token
+ * host-side row lookup `_embd_weights[id]` of kernels/default/model_forward.cpp:87, whose
+ * pointer a captured graph could not change. */
+int frhip_embed_ring(const void *table, int n_rows, int row_bytes, const int32_t *ring, int ring_len,
+                     uint32_t *counter_dev, void *out, frhip_stream s);
+
 /* ---- fused one-token operators ------------------------------------------------ */
 /* Scratch the fused operators need: frhip_decode_workspace_bytes(C, F) bytes,
  * 256-byte aligned, owned by the caller, reusable across calls on one stream. */

@@ -1,0 +1,124 @@
+"""GPU parity tests through the C++ host layer: rwkv::Model("<file>.fr", "hip fp16"|"hip int8")
+against the oracle on the same weights -- the path chat / bench_model take."""
+import importlib
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import pyoracle as po
+from synth import make_model, matrix_indices, quantize_u8
+
+fr = importlib.import_module("faster-rwkv_amd")
+
+L_, C_, F_, V_ = 12, 512, 2048, 4096
+
+
+@pytest.fixture(scope="module")
+def model_files(tmp_path_factory):
+    d = tmp_path_factory.mktemp("fr")
+    params, emb = make_model(4, L_, C_, F_, V_, seed=5)
+    path = str(d / "v4.fr")
+    fr.write_fr(path, "4", L_, C_, F_, 0, params, emb)
+    return path, params, emb
+
+
+def _oracle(params, emb, quant):
+    p = list(params)
+    if quant:
+        for i in matrix_indices(4, L_):
+            p[i] = po.dequant_u8(*quantize_u8(params[i]))
+    return po.Model(4, po.F16, L_, C_, F_, 0, V_, p, emb)
+
+
+@pytest.mark.parametrize("strategy", ["hip fp16", "hip int8"])
+def test_model_run_matches_oracle_over_128_greedy_steps(model_files, strategy):
+    path, params, emb = model_files
+    m = fr.Model(path, strategy)
+    assert (m.n_layer, m.n_embd, m.vocab) == (L_, C_, V_)
+    om = _oracle(params, emb, strategy.endswith("int8"))
+    prompt = np.random.default_rng(42).integers(0, V_, 16)
+    for t in prompt:
+        lh, lo = m.run(int(t)), om.run(int(t))
+    worst = 0.0
+    for step in range(128):
+        worst = max(worst, float(np.abs(lh - lo).max()))
+        th, to = int(np.argmax(lh)), int(np.argmax(lo))
+        assert th == to, "greedy token differs at step %d" % step
+        lh, lo = m.run(th), om.run(to)
+    print(strategy, "worst |dlogit| over 128 steps:", worst, flush=True)
+    assert worst <= 2e-2
+    aa = m.state(11, 1, np.float32)
+    ref = om.state[11 * 5 + 1]
+    assert np.abs(aa - ref).max() <= 5e-3 * np.abs(ref).max()
+    m.close()
+
+
+def test_fused_graph_path_equals_operator_by_operator_path(model_files):
+    path, _, _ = model_files
+    ids = [3, 1000, 77, 77, 4095, 0, 9]
+    m = fr.Model(path, "hip fp16")
+    fused = [m.run(i) for i in ids]
+    m.close()
+    os.environ["FR_HIP_GENERIC"] = "1"
+    try:
+        g = fr.Model(path, "hip fp16")
+        generic = [g.run(i) for i in ids]
+        g.close()
+    finally:
+        del os.environ["FR_HIP_GENERIC"]
+    for a, b in zip(fused, generic):
+        assert np.array_equal(a, b)  # same kernels, same order of arithmetic
+
+
+def test_reset_and_state_file_round_trip(model_files, tmp_path):
+    """tests/test_model.cpp:35-51 (save -> run -> load -> run reproduces) and :93-97."""
+    path, _, _ = model_files
+    m = fr.Model(path, "hip fp16")
+    a = [m.run(i) for i in (1, 2, 3)]
+    m.reset()
+    b = [m.run(i) for i in (1, 2, 3)]
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    sf = str(tmp_path / "state.bin")
+    m.save_state(sf)
+    c = m.run(4)
+    m.run(5)
+    m.load_state(sf)
+    d = m.run(4)
+    assert np.array_equal(c, d)
+    m.close()
+
+
+def test_seq_mode_equals_one_token_steps(model_files):
+    """kernels/default/model_forward_seq.cpp:34-46: Run(ids) == Run(id) for each id."""
+    path, _, _ = model_files
+    ids = [5, 17, 299, 0, 42, 7, 7, 123]
+    m = fr.Model(path, "hip fp16")
+    seq = m.run(ids)
+    m.reset()
+    for i in ids:
+        one = m.run(i)
+    assert np.abs(seq - one).max() <= 2e-2
+    m.close()
+
+
+def test_synthetic_model_and_cpp_greedy_loop():
+    m = fr.Model("synthetic:v=4,L=2,C=256,F=1024,V=1024,seed=7", "hip int8")
+    toks, secs = m.greedy(1, 16)
+    m.reset()
+    again, _ = m.greedy(1, 16)
+    assert np.array_equal(toks, again) and secs > 0
+    assert (toks >= 0).all() and (toks < 1024).all()
+    m.close()
+
+
+def test_bad_arguments_surface_as_exceptions(model_files):
+    path, _, _ = model_files
+    with pytest.raises(fr.FrhipError):
+        fr.Model(path, "hip fp32")
+    m = fr.Model(path, "hip fp16")
+    with pytest.raises(fr.FrhipError):
+        m.run(V_ + 5)
+    m.close()
