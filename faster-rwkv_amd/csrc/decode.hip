@@ -2,13 +2,18 @@
 //
 // The decode step of RWKV is a chain of matrix-vector products separated by cheap
 // elementwise work; each product streams its weight matrix from HBM exactly once,
-// so the whole step is bound by HBM bandwidth.  The kernels here are organised
-// around that:
+// so the whole step is bound by HBM bandwidth and, because a 2048x2048 binary16
+// matrix is only 8 MB (1 us at 8 TB/s), by how fast a launch gets its loads in flight.
+// The kernels are organised around that:
 //   * weights are output-major ([N][K]); a wavefront takes whole rows, each lane
 //     loads 16 contiguous bytes per row chunk, products accumulate in fp32 and are
 //     reduced across lanes with DPP adds.  No partial sums ever leave the wave, so
 //     every elementwise epilogue (sigmoid, WKV update, relu^2, residual) runs in
 //     the lane that owns the output and is fused into the same launch;
+//   * a wave issues the loads of its first batch of rows BEFORE the workgroup's
+//     prologue (weights do not depend on activations), so HBM latency overlaps the
+//     layernorm / token-shift work; with one workgroup per CU most launches are a
+//     single batch per wave, i.e. the whole matrix is requested in the first microsecond;
 //   * the layernorm + token-shift mix that precedes a product is recomputed by
 //     every workgroup into LDS (the activation vector is a few KB and L2-resident),
 //     which removes the separate launches the reference makes for them
@@ -17,6 +22,10 @@
 //     and key of ffn) so that a launch moves tens of MB.
 // One RWKV-4 layer is four launches; the reference issues seventeen
 // (kernels/cuda/att.cu:182-217, ffn.cu:62-87).
+#include <climits>
+#include <cstring>
+#include <type_traits>
+
 #include "device_utils.h"
 #include "frhip_internal.h"
 
@@ -26,6 +35,7 @@ namespace frhip {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / kWave;
+constexpr int kMaxSeg = 4;
 
 struct WMat {
   const unsigned char* data;
@@ -62,8 +72,11 @@ __device__ __forceinline__ LnOut ln_block(const h1* x, const h1* gamma, const h1
   o.active = e0 < C;
   float xf[8];
   float s = 0.f;
+  h8 g, b;
   if (o.active) {
     h8 xv = *reinterpret_cast<const h8*>(x + e0);
+    g = *reinterpret_cast<const h8*>(gamma + e0);
+    b = *reinterpret_cast<const h8*>(beta + e0);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       xf[i] = (float)xv[i];
@@ -83,8 +96,6 @@ __device__ __forceinline__ LnOut ln_block(const h1* x, const h1* gamma, const h1
   var = var > 0.f ? var : 0.f;
   const float inv = 1.0f / sqrtf(var + 1e-5f);
   if (o.active) {
-    h8 g = *reinterpret_cast<const h8*>(gamma + e0);
-    h8 b = *reinterpret_cast<const h8*>(beta + e0);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       h1 n = (h1)((xf[i] - mean) * inv);
@@ -101,46 +112,75 @@ __device__ __forceinline__ h8 mix8(h8 xx, h8 sx, h8 m) {
   return o;
 }
 
-// Rows [r0, r1) of one matrix against one staged vector, R rows in flight per
-// wave; lane j (j < R) receives the finished sum of row n+j and runs the epilogue.
-template <int R, bool U8, class Epi>
-__device__ __forceinline__ void gemv_rows(const WMat& m, const XVec& xv, int r0, int r1, int lane, Epi epi) {
-  const size_t row_bytes = U8 ? (size_t)m.K : 2 * (size_t)m.K;
-  for (int n = r0; n < r1; n += R) {
-    const void* rows[R];
-    XVec xvs[R];
-    RowQ rq[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      int nn = n + r < r1 ? n + r : r1 - 1;  // clamp: surplus slots re-read the last row
-      rows[r] = m.data + (size_t)nn * row_bytes;
-      xvs[r] = xv;
-      if constexpr (U8) {
-        rq[r].c255 = dequant_c255(m.rx[nn]);
-        rq[r].mx = m.mx[nn];
-      }
-    }
-    float acc[R];
-    dot_rows<R, U8>(rows, xvs, rq, m.K, lane, acc);
-    float mine = 0.f;
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      float t = wave_sum(acc[r]);
-      if (lane == r) mine = t;
-    }
-    if (lane < R && n + lane < r1) epi(n + lane, mine);
-  }
-}
-
 // Even split of `total` items over `parts`: part i gets [lo, hi).
 __device__ __forceinline__ void split_even(int total, int parts, int i, int& lo, int& hi) {
   lo = (int)(((long long)total * i) / parts);
   hi = (int)(((long long)total * (i + 1)) / parts);
 }
 
+// ---------------------------------------------------------------------------
+// A batch of R weight rows held in registers: NCH 16-byte chunks per lane per row
+// (lane l owns chunks l, l+64, ...).  load() only issues the loads; dot() consumes
+// them against LDS-resident vectors.  K <= NCH * 64 * (8 | 16) elements.
+// ---------------------------------------------------------------------------
+template <int R, int NCH, bool U8>
+struct RowBatch {
+  using V = typename std::conditional<U8, u32x4, h8>::type;
+  V w[R][NCH];
+
+  __device__ __forceinline__ void load(const void* const (&rows)[R], int nchunk, int lane) {
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+      for (int j = 0; j < NCH; j++) {
+        const int c = lane + j * kWave;
+        if (c < nchunk) w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const V*>(rows[r]) + c);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void dot(const XVec (&xv)[R], const RowQ (&rq)[R], int nchunk, int lane,
+                                      float (&acc)[R]) const {
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+      const int c = lane + j * kWave;
+      if (c < nchunk) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          if constexpr (!U8) {
+            h8 x = reinterpret_cast<const h8*>(xv[r].x)[c];
+            acc[r] = dot8acc(w[r][j], x, acc[r]);
+          } else {
+            // split staging: 8-element groups with even index first, odd ones second,
+            // so consecutive lanes read consecutive 16-byte LDS words
+            const h8* xp = reinterpret_cast<const h8*>(xv[r].x) + c;
+            const h8* ryp = reinterpret_cast<const h8*>(xv[r].ry) + c;
+            const h8* myp = reinterpret_cast<const h8*>(xv[r].my) + c;
+            const h2 c2 = {rq[r].c255, rq[r].c255};
+            const h2 m2 = {rq[r].mx, rq[r].mx};
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+              h8 x = xp[hh * nchunk], ry = ryp[hh * nchunk], my = myp[hh * nchunk];
+              uint32_t w0 = w[r][j][2 * hh], w1 = w[r][j][2 * hh + 1];
+              acc[r] = dot2acc(dequant_pair<0>(w0, c2, m2, ry.s01, my.s01), x.s01, acc[r]);
+              acc[r] = dot2acc(dequant_pair<1>(w0, c2, m2, ry.s23, my.s23), x.s23, acc[r]);
+              acc[r] = dot2acc(dequant_pair<0>(w1, c2, m2, ry.s45, my.s45), x.s45, acc[r]);
+              acc[r] = dot2acc(dequant_pair<1>(w1, c2, m2, ry.s67, my.s67), x.s67, acc[r]);
+            }
+          }
+        }
+      }
+    }
+  }
+};
+
 // ===========================================================================
 // att, front half:  LN -> mix -> k,v,r products -> sigmoid -> WKV-4 update
 //                   -> r * wkv                    (kernels/cuda/att.cu:183-211)
+// One channel = three rows (one of each matrix); the wave that owns a channel owns
+// its recurrent state.
 // ===========================================================================
 struct AttFrontV4 {
   int C;
@@ -151,15 +191,30 @@ struct AttFrontV4 {
   float *aa_out, *bb_out, *pp_out;
 };
 
-template <bool U8>
+template <int NCH, bool U8>
 __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float red[kWaves];
   const int C = a.C;
+  const int nchunk = U8 ? (C >> 4) : (C >> 3);
   h1* kx = reinterpret_cast<h1*>(smem);
   h1* vx = kx + C;
   h1* rx = vx + C;
   h1* qv = rx + C;  // uint8 only: ry,my of kw ; ry,my of vw ; ry,my of rw
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int gw = blockIdx.x * kWaves + threadIdx.x / kWave;
+  int c0, c1;
+  split_even(C, gridDim.x * kWaves, gw, c0, c1);
+  const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
+
+  RowBatch<3, NCH, U8> cur;
+  // recurrent state and time parameters of the first channel, requested before anything else
+  float st_tf = 0.f, st_td = 0.f, st_pp = 0.f, st_aa = 0.f, st_bb = 0.f;
+  if (c0 < c1) {
+    const void* rows[3] = {a.kw.data + c0 * row_bytes, a.vw.data + c0 * row_bytes, a.rw.data + c0 * row_bytes};
+    cur.load(rows, nchunk, lane);
+  }
 
   LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, C, red);
   if (ln.active) {
@@ -181,14 +236,14 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   }
   __syncthreads();
 
-  const int lane = threadIdx.x & (kWave - 1);
-  const int gw = blockIdx.x * kWaves + threadIdx.x / kWave;
-  int c0, c1;
-  split_even(C, gridDim.x * kWaves, gw, c0, c1);
-  const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
+  const XVec xv[3] = {{kx, qv + 0 * C, qv + 1 * C}, {vx, qv + 2 * C, qv + 3 * C}, {rx, qv + 4 * C, qv + 5 * C}};
   for (int n = c0; n < c1; n++) {
-    const void* rows[3] = {a.kw.data + n * row_bytes, a.vw.data + n * row_bytes, a.rw.data + n * row_bytes};
-    XVec xv[3] = {{kx, qv + 0 * C, qv + 1 * C}, {vx, qv + 2 * C, qv + 3 * C}, {rx, qv + 4 * C, qv + 5 * C}};
+    RowBatch<3, NCH, U8> nxt;
+    if (n + 1 < c1) {
+      const void* rows[3] = {a.kw.data + (n + 1) * row_bytes, a.vw.data + (n + 1) * row_bytes,
+                             a.rw.data + (n + 1) * row_bytes};
+      nxt.load(rows, nchunk, lane);
+    }
     RowQ rq[3];
     if constexpr (U8) {
       rq[0] = {dequant_c255(a.kw.rx[n]), a.kw.mx[n]};
@@ -196,22 +251,25 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       rq[2] = {dequant_c255(a.rw.rx[n]), a.rw.mx[n]};
     }
     float acc[3];
-    dot_rows<3, U8>(rows, xv, rq, C, lane, acc);
+    cur.dot(xv, rq, nchunk, lane, acc);
     const float k = wave_sum(acc[0]);
     const float v = wave_sum(acc[1]);
     const float rr = wave_sum(acc[2]);
     if (lane == 0) {
       // kernels/cuda/att.cu:30-62 (WkvForwardOne), r already passed through sigmoid (:203)
+      {
+        st_tf = a.tf[n]; st_td = a.td[n]; st_pp = a.pp[n]; st_aa = a.aa[n]; st_bb = a.bb[n];
+      }
       const h1 r = sigmoid_h((h1)rr);
-      float ww = a.tf[n] + k;
-      const float pp_ = a.pp[n];
+      float ww = st_tf + k;
+      const float pp_ = st_pp;
       float p_ = (pp_ > ww) ? pp_ : ww;
       float e1 = expf(pp_ - p_);
       float e2 = expf(ww - p_);
-      const float aa_ = a.aa[n], bb_ = a.bb[n];
+      const float aa_ = st_aa, bb_ = st_bb;
       const float wkv = (e1 * aa_ + e2 * v) / (e1 * bb_ + e2);
       a.rwkv_out[n] = r * (h1)wkv;
-      ww = a.td[n] + pp_;
+      ww = st_td + pp_;
       p_ = (ww > k) ? ww : k;
       e1 = expf(ww - p_);
       e2 = expf(k - p_);
@@ -219,175 +277,194 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       a.bb_out[n] = e1 * bb_ + e2;
       a.pp_out[n] = p_;
     }
+    if (n + 1 < c1) cur = nxt;
   }
 }
 
 // ===========================================================================
-// Generic "stage a vector, stream rows, epilogue per output" kernels
+// The general row-streaming kernel: up to four matrices ("segments") in one launch,
+// each with its own staged activation vector and per-output epilogue.  Global row g
+// belongs to the segment s with start[s] <= g < start[s+1].
 // ===========================================================================
-// att, back half: out = rwkv . Wo ; x_out = x + out     (att.cu:213-215)
-struct AttOutV4 {
-  int C;
-  const h1 *rwkv, *x;
-  WMat ow;
-  h1* x_out;
+enum Prologue : int {
+  P_COPY = 0,   // stage vec0 from global memory
+  P_LN = 1,     // stage LN(x)
+  P_LN_MIX = 2  // stage mix(LN(x), sx, mix[i]) for i < nvec; workgroup 0 writes LN(x) to xx_out
 };
 
-template <int R, bool U8>
-__global__ __launch_bounds__(kThreads) void att_out_kernel(AttOutV4 a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int K = a.ow.K;
-  h1* xs = reinterpret_cast<h1*>(smem);
-  stage_vec<U8>(xs, a.rwkv, K);
-  if constexpr (U8) {
-    stage_vec<true>(xs + K, a.ow.ry, K);
-    stage_vec<true>(xs + 2 * K, a.ow.my, K);
-  }
-  __syncthreads();
-  const int lane = threadIdx.x & (kWave - 1);
-  int r0, r1;
-  split_even(a.ow.N, gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, r0, r1);
-  XVec xv = {xs, xs + K, xs + 2 * K};
-  gemv_rows<R, U8>(a.ow, xv, r0, r1, lane, [&](int n, float sum) { a.x_out[n] = a.x[n] + (h1)sum; });
-}
-
-// ffn, front half: LN -> mix -> r = sigmoid(rx.Wr) ; vx = relu(kx.Wk)^2   (ffn.cu:66-81)
-struct FfnFront {
-  int C, F;
-  const h1 *x, *sx, *ln_w, *ln_b, *mk, *mr;
-  WMat kw, rw;
-  h1 *xx_out, *r_out, *vx_out;
+enum Epilogue : int {
+  E_STORE_F16 = 0,  // out_h[n] = h(sum)
+  E_STORE_F32 = 1,  // out_f[n] = sum
+  E_RESIDUAL = 2,   // out_h[n] = x[n] + h(sum)                        att.cu:213-215
+  E_SIGMOID = 3,    // out_h[n] = sigmoid(h(sum))                      ffn.cu:78-79
+  E_RELU2 = 4,      // out_h[n] = relu(h(sum))^2                       ffn.cu:80-81
+  E_FFN_OUT = 5,    // out_h[n] = fma(h(sum), r[n], x[n]) [/ 2]        ffn.cu:82-85, model_forward.cpp:173-175
+  E_LOGITS = 6,     // out_f[n] = float(h(sum))                        model_forward.cpp:184-188
+  E_SILU = 7        // out_h[n] = silu(h(sum))                         att.cu:289-290
 };
 
-template <int R, bool U8>
-__global__ __launch_bounds__(kThreads) void ffn_front_kernel(FfnFront a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ float red[kWaves];
-  const int C = a.C, F = a.F;
-  h1* kx = reinterpret_cast<h1*>(smem);
-  h1* rx = kx + C;
-  h1* qv = rx + C;  // uint8 only: ry,my of rw ; ry,my of kw  (all [C])
-  LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, C, red);
-  if (ln.active) {
-    const int e0 = threadIdx.x * 8;
-    h8 sx = *reinterpret_cast<const h8*>(a.sx + e0);
-    const int pos = stage_pos<U8>(threadIdx.x, C);
-    reinterpret_cast<h8*>(kx)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mk + e0));
-    reinterpret_cast<h8*>(rx)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mr + e0));
-    if (blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
-  }
-  if constexpr (U8) {
-    stage_vec<true>(qv + 0 * C, a.rw.ry, C);
-    stage_vec<true>(qv + 1 * C, a.rw.my, C);
-    stage_vec<true>(qv + 2 * C, a.kw.ry, C);
-    stage_vec<true>(qv + 3 * C, a.kw.my, C);
-  }
-  __syncthreads();
-  const int lane = threadIdx.x & (kWave - 1);
-  int g0, g1;  // rows [0,C) are receptance rows, [C, C+F) key rows
-  split_even(C + F, gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, g0, g1);
-  if (g0 < C) {
-    XVec xv = {rx, qv + 0 * C, qv + 1 * C};
-    gemv_rows<R, U8>(a.rw, xv, g0, g1 < C ? g1 : C, lane,
-                     [&](int n, float sum) { a.r_out[n] = sigmoid_h((h1)sum); });
-  }
-  if (g1 > C) {
-    XVec xv = {kx, qv + 2 * C, qv + 3 * C};
-    gemv_rows<R, U8>(a.kw, xv, (g0 > C ? g0 : C) - C, g1 - C, lane, [&](int n, float sum) {
-      h1 t = (h1)sum;  // ffn.cu:41-51
-      a.vx_out[n] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
-    });
-  }
-}
+struct Seg {
+  WMat w;
+  int vec;  // which staged vector this segment multiplies
+  int epi;
+  void* out;
+};
 
-// ffn, back half: out = vx.Wv ; x_out = fma(out, r, x) [; x_out /= 2]   (ffn.cu:82-85)
-struct FfnOut {
-  int C, F;
-  const h1 *vx, *r, *x;
-  WMat vw;
-  h1* x_out;
+struct RowsArgs {
+  int K;          // length of every staged vector == K of every segment
+  int nseg, nvec; // segments, staged vectors
+  int prologue;
+  int start[kMaxSeg + 1];  // first global row of each segment; start[nseg] = total rows
+  Seg seg[kMaxSeg];
+  // prologue inputs
+  const h1* vec0;                      // P_COPY
+  const h1 *x, *sx, *ln_w, *ln_b;      // P_LN, P_LN_MIX
+  const h1* mix[kMaxSeg];              // P_LN_MIX
+  h1* xx_out;                          // P_LN_MIX
+  // epilogue inputs
+  const h1* res_x;  // E_RESIDUAL, E_FFN_OUT
+  const h1* res_r;  // E_FFN_OUT
   int div2;
 };
 
-template <int R, bool U8>
-__global__ __launch_bounds__(kThreads) void ffn_out_kernel(FfnOut a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int K = a.vw.K;
-  h1* xs = reinterpret_cast<h1*>(smem);
-  stage_vec<U8>(xs, a.vx, K);
-  if constexpr (U8) {
-    stage_vec<true>(xs + K, a.vw.ry, K);
-    stage_vec<true>(xs + 2 * K, a.vw.my, K);
+__device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, int n, float sum, h1 ex, h1 er) {
+  switch (sg.epi) {
+    case E_STORE_F16: static_cast<h1*>(sg.out)[n] = (h1)sum; break;
+    case E_STORE_F32: static_cast<float*>(sg.out)[n] = sum; break;
+    case E_RESIDUAL: static_cast<h1*>(sg.out)[n] = a.res_x[n] + (h1)sum; break;
+    case E_SIGMOID: static_cast<h1*>(sg.out)[n] = sigmoid_h((h1)sum); break;
+    case E_RELU2: {
+      h1 t = (h1)sum;
+      static_cast<h1*>(sg.out)[n] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
+      break;
+    }
+    case E_FFN_OUT: {
+      h1 o = __builtin_fmaf16((h1)sum, a.res_r[n], a.res_x[n]);  // __hfma: one rounding
+      if (a.div2) o = o / (h1)2.0f;
+      static_cast<h1*>(sg.out)[n] = o;
+      break;
+    }
+    case E_LOGITS: static_cast<float*>(sg.out)[n] = (float)(h1)sum; break;
+    case E_SILU: static_cast<h1*>(sg.out)[n] = silu_h((h1)sum); break;
+    default: break;
   }
-  __syncthreads();
-  const int lane = threadIdx.x & (kWave - 1);
-  int r0, r1;
-  split_even(a.vw.N, gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, r0, r1);
-  XVec xv = {xs, xs + K, xs + 2 * K};
-  gemv_rows<R, U8>(a.vw, xv, r0, r1, lane, [&](int n, float sum) {
-    h1 o = __builtin_fmaf16((h1)sum, a.r[n], a.x[n]);       // __hfma, one rounding
-    if (a.div2) o = o / (h1)2.0f;                           // model_forward.cpp:173-175
-    a.x_out[n] = o;
-  });
 }
 
-// head: LN(ln_out) -> x.Whead -> half -> fp32   (model_forward.cpp:180-188)
-struct Head {
-  int C;
-  const h1 *x, *ln_w, *ln_b;
-  WMat hw;
-  float* logits;
-};
-
-template <int R, bool U8>
-__global__ __launch_bounds__(kThreads) void head_kernel(Head a) {
+// MULTI = a wave has several batches: two batches live in registers and alternate, the
+// loads of one in flight while the other is consumed.
+template <int R, int NCH, bool U8, bool MULTI>
+__global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float red[kWaves];
-  const int C = a.C;
-  h1* xs = reinterpret_cast<h1*>(smem);
-  LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, C, red);
-  if (ln.active) reinterpret_cast<h8*>(xs)[stage_pos<U8>(threadIdx.x, C)] = ln.xx;
+  const int K = a.K;
+  const int nchunk = U8 ? (K >> 4) : (K >> 3);
+  const size_t row_bytes = U8 ? (size_t)K : 2 * (size_t)K;
+  h1* vecs = reinterpret_cast<h1*>(smem);   // nvec staged activation vectors
+  h1* qv = vecs + (size_t)a.nvec * K;       // uint8: (ry, my) per segment
+
+  const int lane = threadIdx.x & (kWave - 1);
+  // The concatenated row space of all segments is split evenly over the waves of the grid;
+  // global row g belongs to the segment s with start[s] <= g < start[s+1].
+  int g0, g1;
+  split_even(a.start[a.nseg], gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, g0, g1);
+
+  struct Meta {
+    int seg[R], loc[R];
+    h1 ex, er;  // epilogue operands of the row this lane finishes (lane < R)
+  };
+  // locate the rows of the batch starting at global row g and issue their loads
+  auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int g) {
+    const void* rows[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const int gg = g + r < g1 ? g + r : g1 - 1;  // surplus slots re-read the last row
+      int sg = 0;
+#pragma unroll
+      for (int i = 1; i < kMaxSeg; i++) sg += (i < a.nseg && gg >= a.start[i]) ? 1 : 0;
+      m.seg[r] = sg;
+      m.loc[r] = gg - a.start[sg];
+      rows[r] = a.seg[sg].w.data + (size_t)m.loc[r] * row_bytes;
+    }
+    b.load(rows, nchunk, lane);
+    m.ex = (h1)0.0f;
+    m.er = (h1)0.0f;
+  };
+  auto consume = [&](const RowBatch<R, NCH, U8>& b, const Meta& m, int g) {
+    XVec xv[R];
+    RowQ rq[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const Seg& sg = a.seg[m.seg[r]];
+      xv[r].x = vecs + (size_t)sg.vec * K;
+      xv[r].ry = qv + (size_t)(2 * m.seg[r]) * K;
+      xv[r].my = qv + (size_t)(2 * m.seg[r] + 1) * K;
+      if constexpr (U8) {
+        rq[r].c255 = dequant_c255(sg.w.rx[m.loc[r]]);
+        rq[r].mx = sg.w.mx[m.loc[r]];
+      }
+    }
+    float acc[R];
+    b.dot(xv, rq, nchunk, lane, acc);
+    float mine = 0.f;
+    int my_seg = 0, my_loc = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const float t = wave_sum(acc[r]);
+      if (lane == r) {
+        mine = t;
+        my_seg = m.seg[r];
+        my_loc = m.loc[r];
+      }
+    }
+    if (lane < R && g + lane < g1) run_epilogue(a, a.seg[my_seg], my_loc, mine, m.ex, m.er);
+  };
+
+  RowBatch<R, NCH, U8> A;
+  Meta mA;
+  if (g0 < g1) fetch(A, mA, g0);
+
+  // ---- prologue: stage the activation vector(s) in LDS ----
+  if (a.prologue == P_COPY) {
+    stage_vec<U8>(vecs, a.vec0, K);
+  } else {
+    LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, K, red);
+    if (ln.active) {
+      const int e0 = threadIdx.x * 8;
+      const int pos = stage_pos<U8>(threadIdx.x, K);
+      if (a.prologue == P_LN) {
+        reinterpret_cast<h8*>(vecs)[pos] = ln.xx;
+      } else {
+        h8 sx = *reinterpret_cast<const h8*>(a.sx + e0);
+        for (int i = 0; i < a.nvec; i++)
+          reinterpret_cast<h8*>(vecs + (size_t)i * K)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mix[i] + e0));
+        if (blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
+      }
+    }
+  }
   if constexpr (U8) {
-    stage_vec<true>(xs + C, a.hw.ry, C);
-    stage_vec<true>(xs + 2 * C, a.hw.my, C);
+    for (int s = 0; s < a.nseg; s++) {
+      stage_vec<true>(qv + (size_t)(2 * s) * K, a.seg[s].w.ry, K);
+      stage_vec<true>(qv + (size_t)(2 * s + 1) * K, a.seg[s].w.my, K);
+    }
   }
   __syncthreads();
-  const int lane = threadIdx.x & (kWave - 1);
-  int r0, r1;
-  split_even(a.hw.N, gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, r0, r1);
-  XVec xv = {xs, xs + C, xs + 2 * C};
-  gemv_rows<R, U8>(a.hw, xv, r0, r1, lane, [&](int n, float sum) { a.logits[n] = (float)(h1)sum; });
-}
 
-// plain matmul, vector x matrix   (kernels/cuda/matmul.cpp:105-109)
-struct Gemv {
-  const h1* x;
-  WMat w;
-  void* y;
-  int out_f32;
-};
-
-template <int R, bool U8>
-__global__ __launch_bounds__(kThreads) void gemv_kernel(Gemv a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int K = a.w.K;
-  h1* xs = reinterpret_cast<h1*>(smem);
-  stage_vec<U8>(xs, a.x, K);
-  if constexpr (U8) {
-    stage_vec<true>(xs + K, a.w.ry, K);
-    stage_vec<true>(xs + 2 * K, a.w.my, K);
+  if constexpr (!MULTI) {
+    if (g0 < g1) consume(A, mA, g0);  // the host guarantees g1 - g0 <= R
+  } else {
+    RowBatch<R, NCH, U8> B;
+    Meta mB;
+    int g = g0;
+    while (g < g1) {
+      if (g + R < g1) fetch(B, mB, g + R);
+      consume(A, mA, g);
+      g += R;
+      if (g >= g1) break;
+      if (g + R < g1) fetch(A, mA, g + R);
+      consume(B, mB, g);
+      g += R;
+    }
   }
-  __syncthreads();
-  const int lane = threadIdx.x & (kWave - 1);
-  int r0, r1;
-  split_even(a.w.N, gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, r0, r1);
-  XVec xv = {xs, xs + K, xs + 2 * K};
-  gemv_rows<R, U8>(a.w, xv, r0, r1, lane, [&](int n, float sum) {
-    if (a.out_f32)
-      static_cast<float*>(a.y)[n] = sum;
-    else
-      static_cast<h1*>(a.y)[n] = (h1)sum;
-  });
 }
 
 // ---------------------------------------------------------------------------
@@ -415,50 +492,139 @@ static int check_vec(const void* p, const char* what) {
   return 0;
 }
 
-#define FR_TRY(expr)            \
-  do {                          \
-    int _e = (expr);            \
-    if (_e != 0) return _e;     \
+#define FR_TRY(expr)        \
+  do {                      \
+    int _e = (expr);        \
+    if (_e != 0) return _e; \
   } while (0)
 
 static int check_embd(int C) {
-  if (C <= 0 || C % 16 != 0 || C > 8 * kThreads) return set_error(FRHIP_ESHAPE, "n_embd must be a multiple of 16 and at most 4096");
+  if (C <= 0 || C % 16 != 0 || C > 8 * kThreads)
+    return set_error(FRHIP_ESHAPE, "n_embd must be a multiple of 16 and at most 4096");
   return 0;
 }
-
-// Rows in flight per wave: all of a wave's rows when that is few, else 4.
-static int pick_r(long rows, int grid, bool u8) {
-  long waves = (long)grid * kWaves;
-  long per = (rows + waves - 1) / waves;
-  int cap = u8 ? 4 : 6;
-  if (per <= cap) return (int)(per < 1 ? 1 : per);
-  return 4;
-}
-
-#define DISPATCH_R_U8(KERNEL, R, U8, GRID, LDS, STREAM, ARGS)                                          \
-  do {                                                                                                 \
-    if (U8) {                                                                                          \
-      switch (R) {                                                                                     \
-        case 1: hipLaunchKernelGGL((KERNEL<1, true>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        case 2: hipLaunchKernelGGL((KERNEL<2, true>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        case 3: hipLaunchKernelGGL((KERNEL<3, true>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        default: hipLaunchKernelGGL((KERNEL<4, true>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-      }                                                                                                \
-    } else {                                                                                           \
-      switch (R) {                                                                                     \
-        case 1: hipLaunchKernelGGL((KERNEL<1, false>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        case 2: hipLaunchKernelGGL((KERNEL<2, false>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        case 3: hipLaunchKernelGGL((KERNEL<3, false>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        case 5: hipLaunchKernelGGL((KERNEL<5, false>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        case 6: hipLaunchKernelGGL((KERNEL<6, false>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-        default: hipLaunchKernelGGL((KERNEL<4, false>), dim3(GRID), dim3(kThreads), LDS, STREAM, ARGS); break; \
-      }                                                                                                \
-    }                                                                                                  \
-  } while (0)
 
 static int check_lds(size_t bytes) {
   if (bytes > 64 * 1024) return set_error(FRHIP_ESHAPE, "vector operands exceed 64 KB of LDS");
   return 0;
+}
+
+// Chunks (16 bytes per lane) a lane holds per row.
+static int chunks_per_lane(int K, bool u8) {
+  const int nchunk = u8 ? K / 16 : K / 8;
+  return (nchunk + kWave - 1) / kWave;
+}
+
+// Supported register tilings.  NCH is rounded up to one of these; R is then chosen so
+// that a wave's rows fit in one batch when that needs at most kMaxLoads loads per lane.
+static const int kNchSet[] = {1, 2, 3, 4, 5, 8, 9, 16, 18};
+constexpr int kMaxLoads = 32;
+
+static int round_nch(int nch) {
+  for (int v : kNchSet)
+    if (nch <= v) return v;
+  return -1;
+}
+
+// Rows in flight per wave.  When all rows of a wave fit in kMaxLoads loads per lane they
+// form one batch (multi = false); otherwise batches of at most kMaxLoads/2 loads alternate
+// between two register sets.
+static int pick_r(const RowsArgs& a, int grid, int nch, bool* multi) {
+  const long waves = (long)grid * kWaves;
+  long per = ((long)a.start[a.nseg] + waves - 1) / waves;  // most rows any wave gets
+  if (per < 1) per = 1;
+  int rmax = kMaxLoads / nch;
+  if (rmax < 1) rmax = 1;
+  if (rmax > 6) rmax = 6;
+  if (per <= rmax) {
+    *multi = false;
+    return (int)per;
+  }
+  *multi = true;
+  int r = (kMaxLoads / 2) / nch;
+  if (r < 1) r = 1;
+  if (r > 4) r = 4;
+  return r;
+}
+
+// false when the (R, NCH, MULTI) tiling is not compiled (pick_r never asks for one that is not)
+template <int R, int NCH>
+static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
+  if (!multi) {
+    if constexpr (R * NCH <= kMaxLoads || R == 1) {
+      if (u8)
+        hipLaunchKernelGGL((rows_kernel<R, NCH, true, false>), dim3(grid), dim3(kThreads), lds, st, a);
+      else
+        hipLaunchKernelGGL((rows_kernel<R, NCH, false, false>), dim3(grid), dim3(kThreads), lds, st, a);
+      return true;
+    }
+  } else {
+    if constexpr ((R * NCH <= kMaxLoads / 2 && R <= 4) || R == 1) {
+      if (u8)
+        hipLaunchKernelGGL((rows_kernel<R, NCH, true, true>), dim3(grid), dim3(kThreads), lds, st, a);
+      else
+        hipLaunchKernelGGL((rows_kernel<R, NCH, false, true>), dim3(grid), dim3(kThreads), lds, st, a);
+      return true;
+    }
+  }
+  return false;
+}
+
+template <int NCH>
+static bool launch_rows_n(int R, bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
+  switch (R) {
+    case 1: return launch_rows_rn<1, NCH>(u8, multi, grid, lds, st, a);
+    case 2: return launch_rows_rn<2, NCH>(u8, multi, grid, lds, st, a);
+    case 3: return launch_rows_rn<3, NCH>(u8, multi, grid, lds, st, a);
+    case 4: return launch_rows_rn<4, NCH>(u8, multi, grid, lds, st, a);
+    case 5: return launch_rows_rn<5, NCH>(u8, multi, grid, lds, st, a);
+    case 6: return launch_rows_rn<6, NCH>(u8, multi, grid, lds, st, a);
+    default: return false;
+  }
+}
+
+static int launch_rows(const RowsArgs& a, bool u8, hipStream_t st, const char* what) {
+  const int nch = round_nch(chunks_per_lane(a.K, u8));
+  if (nch < 0) return set_error(FRHIP_ESHAPE, "K is too large for the row-streaming kernel (max 9216 fp16 / 18432 uint8)");
+  const int grid = decode_grid();
+  bool multi = false;
+  const int R = pick_r(a, grid, nch, &multi);
+  const size_t lds = 2 * (size_t)a.K * (a.nvec + (u8 ? 2 * a.nseg : 0));
+  FR_TRY(check_lds(lds));
+  bool ok = false;
+  switch (nch) {
+    case 1: ok = launch_rows_n<1>(R, u8, multi, grid, lds, st, a); break;
+    case 2: ok = launch_rows_n<2>(R, u8, multi, grid, lds, st, a); break;
+    case 3: ok = launch_rows_n<3>(R, u8, multi, grid, lds, st, a); break;
+    case 4: ok = launch_rows_n<4>(R, u8, multi, grid, lds, st, a); break;
+    case 5: ok = launch_rows_n<5>(R, u8, multi, grid, lds, st, a); break;
+    case 8: ok = launch_rows_n<8>(R, u8, multi, grid, lds, st, a); break;
+    case 9: ok = launch_rows_n<9>(R, u8, multi, grid, lds, st, a); break;
+    case 16: ok = launch_rows_n<16>(R, u8, multi, grid, lds, st, a); break;
+    case 18: ok = launch_rows_n<18>(R, u8, multi, grid, lds, st, a); break;
+    default: break;
+  }
+  if (!ok) return set_error(FRHIP_ESHAPE, "row-streaming kernel: no compiled tiling for this shape");
+  return check_launch(what);
+}
+
+static RowsArgs empty_args(int K) {
+  RowsArgs a;
+  memset(&a, 0, sizeof(a));
+  a.K = K;
+  for (int i = 0; i <= kMaxSeg; i++) a.start[i] = INT_MAX;
+  return a;
+}
+
+static void add_seg(RowsArgs& a, const frhip_weight* w, int vec, int epi, void* out) {
+  const int s = a.nseg;
+  a.start[s] = s == 0 ? 0 : a.start[s];
+  a.seg[s].w = to_wmat(w);
+  a.seg[s].vec = vec;
+  a.seg[s].epi = epi;
+  a.seg[s].out = out;
+  a.start[s + 1] = a.start[s] + w->N;
+  a.nseg = s + 1;
 }
 
 }  // namespace frhip
@@ -466,7 +632,7 @@ static int check_lds(size_t bytes) {
 using namespace frhip;
 
 extern "C" size_t frhip_decode_workspace_bytes(int C, int F) {
-  // rwkv [C] | r [C] | vx [F] | x_mid [C]   (binary16), each 256-byte aligned
+  // rwkv [C] | r [C] | x_mid [C] | vx [F]   (binary16), each 256-byte aligned
   auto al = [](size_t n) { return (n + 255) / 256 * 256; };
   if (C <= 0 || F <= 0) return 0;
   return al(2 * (size_t)C) * 3 + al(2 * (size_t)F);
@@ -476,7 +642,7 @@ namespace {
 struct Workspace {
   h1 *rwkv, *r, *vx, *xmid;
 };
-Workspace carve(void* ws, int C, int F) {
+Workspace carve(void* ws, int C) {
   auto al = [](size_t n) { return (n + 255) / 256 * 256; };
   unsigned char* p = static_cast<unsigned char*>(ws);
   Workspace w;
@@ -487,7 +653,6 @@ Workspace carve(void* ws, int C, int F) {
   w.xmid = reinterpret_cast<h1*>(p);
   p += al(2 * (size_t)C);
   w.vx = reinterpret_cast<h1*>(p);
-  (void)F;
   return w;
 }
 }  // namespace
@@ -518,7 +683,7 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   FR_TRY(check_weight(ow, C, C));
   if (kw->dtype != vw->dtype || kw->dtype != rw->dtype) return set_error(FRHIP_EINVAL, "att: key/value/receptance dtypes differ");
   hipStream_t st = static_cast<hipStream_t>(s);
-  Workspace w = carve(workspace, C, 16);
+  Workspace w = carve(workspace, C);
   const int grid = decode_grid();
 
   AttFrontV4 a;
@@ -530,21 +695,31 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   a.xx_out = (h1*)xx_out; a.rwkv_out = w.rwkv;
   a.aa_out = aa_out; a.bb_out = bb_out; a.pp_out = pp_out;
   const bool u8 = kw->dtype == FRHIP_U8;
-  size_t lds = 2 * (size_t)C * (u8 ? 9 : 3);
+  const size_t lds = 2 * (size_t)C * (u8 ? 9 : 3);
   FR_TRY(check_lds(lds));
-  if (u8)
-    hipLaunchKernelGGL(att_front_v4_kernel<true>, dim3(grid), dim3(kThreads), lds, st, a);
-  else
-    hipLaunchKernelGGL(att_front_v4_kernel<false>, dim3(grid), dim3(kThreads), lds, st, a);
+  const int nch = chunks_per_lane(C, u8);  // C <= 4096: at most 8 (fp16) or 4 (uint8)
+#define FR_ATT_FRONT(N)                                                                                   \
+  do {                                                                                                    \
+    if (u8)                                                                                               \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, true>), dim3(grid), dim3(kThreads), lds, st, a);         \
+    else                                                                                                  \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, false>), dim3(grid), dim3(kThreads), lds, st, a);        \
+  } while (0)
+  if (nch <= 1) FR_ATT_FRONT(1);
+  else if (nch == 2) FR_ATT_FRONT(2);
+  else if (nch <= 4) FR_ATT_FRONT(4);
+  else if (nch == 5) FR_ATT_FRONT(5);
+  else FR_ATT_FRONT(8);
+#undef FR_ATT_FRONT
   FR_TRY(check_launch("att_front_v4"));
 
-  AttOutV4 b;
-  b.C = C; b.rwkv = w.rwkv; b.x = (const h1*)x; b.ow = to_wmat(ow); b.x_out = (h1*)x_out;
-  const bool ou8 = ow->dtype == FRHIP_U8;
-  lds = 2 * (size_t)C * (ou8 ? 3 : 1);
-  const int R = pick_r(C, grid, ou8);
-  DISPATCH_R_U8(att_out_kernel, R, ou8, grid, lds, st, b);
-  return check_launch("att_out");
+  RowsArgs b = empty_args(C);
+  b.prologue = P_COPY;
+  b.nvec = 1;
+  b.vec0 = w.rwkv;
+  b.res_x = (const h1*)x;
+  add_seg(b, ow, 0, E_RESIDUAL, x_out);
+  return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_out");
 }
 
 extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const void* ln_w, const void* ln_b,
@@ -568,31 +743,28 @@ extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const 
   FR_TRY(check_weight(rw, C, C));
   if (kw->dtype != rw->dtype) return set_error(FRHIP_EINVAL, "ffn: key/receptance dtypes differ");
   hipStream_t st = static_cast<hipStream_t>(s);
-  Workspace w = carve(workspace, C, F);
-  const int grid = decode_grid();
+  Workspace w = carve(workspace, C);
 
-  FfnFront a;
-  a.C = C; a.F = F;
+  RowsArgs a = empty_args(C);
+  a.prologue = P_LN_MIX;
+  a.nvec = 2;
   a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
-  a.mk = (const h1*)k_mix; a.mr = (const h1*)r_mix;
-  a.kw = to_wmat(kw); a.rw = to_wmat(rw);
-  a.xx_out = (h1*)xx_out; a.r_out = w.r; a.vx_out = w.vx;
-  const bool u8 = kw->dtype == FRHIP_U8;
-  size_t lds = 2 * (size_t)C * (u8 ? 6 : 2);
-  FR_TRY(check_lds(lds));
-  int R = pick_r((long)C + F, grid, u8);
-  DISPATCH_R_U8(ffn_front_kernel, R, u8, grid, lds, st, a);
-  FR_TRY(check_launch("ffn_front"));
+  a.mix[0] = (const h1*)r_mix;
+  a.mix[1] = (const h1*)k_mix;
+  a.xx_out = (h1*)xx_out;
+  add_seg(a, rw, 0, E_SIGMOID, w.r);
+  add_seg(a, kw, 1, E_RELU2, w.vx);
+  FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "ffn_front"));
 
-  FfnOut b;
-  b.C = C; b.F = F; b.vx = w.vx; b.r = w.r; b.x = (const h1*)x; b.vw = to_wmat(vw);
-  b.x_out = (h1*)x_out; b.div2 = post_div2 ? 1 : 0;
-  const bool vu8 = vw->dtype == FRHIP_U8;
-  lds = 2 * (size_t)F * (vu8 ? 3 : 1);
-  FR_TRY(check_lds(lds));
-  R = pick_r(C, grid, vu8);
-  DISPATCH_R_U8(ffn_out_kernel, R, vu8, grid, lds, st, b);
-  return check_launch("ffn_out");
+  RowsArgs b = empty_args(F);
+  b.prologue = P_COPY;
+  b.nvec = 1;
+  b.vec0 = w.vx;
+  b.res_x = (const h1*)x;
+  b.res_r = w.r;
+  b.div2 = post_div2 ? 1 : 0;
+  add_seg(b, vw, 0, E_FFN_OUT, x_out);
+  return launch_rows(b, vw->dtype == FRHIP_U8, st, "ffn_out");
 }
 
 extern "C" int frhip_head(int C, const void* x, const void* ln_w, const void* ln_b, const frhip_weight* head,
@@ -603,16 +775,12 @@ extern "C" int frhip_head(int C, const void* x, const void* ln_w, const void* ln
   FR_TRY(check_vec(ln_b, "ln_b is null or misaligned"));
   if (!logits) return set_error(FRHIP_EINVAL, "logits is null");
   FR_TRY(check_weight(head, C, 0));
-  Head a;
-  a.C = C; a.x = (const h1*)x; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
-  a.hw = to_wmat(head); a.logits = logits;
-  const bool u8 = head->dtype == FRHIP_U8;
-  const int grid = decode_grid();
-  size_t lds = 2 * (size_t)C * (u8 ? 3 : 1);
-  FR_TRY(check_lds(lds));
-  const int R = pick_r(head->N, grid, u8);
-  DISPATCH_R_U8(head_kernel, R, u8, grid, lds, static_cast<hipStream_t>(s), a);
-  return check_launch("head");
+  RowsArgs a = empty_args(C);
+  a.prologue = P_LN;
+  a.nvec = 1;
+  a.x = (const h1*)x; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+  add_seg(a, head, 0, E_LOGITS, logits);
+  return launch_rows(a, head->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "head");
 }
 
 extern "C" int frhip_gemv(const void* x, const frhip_weight* w, void* y, int out_dtype, frhip_stream s) {
@@ -620,13 +788,10 @@ extern "C" int frhip_gemv(const void* x, const frhip_weight* w, void* y, int out
   if (!y) return set_error(FRHIP_EINVAL, "y is null");
   if (out_dtype != FRHIP_F16 && out_dtype != FRHIP_F32) return set_error(FRHIP_EINVAL, "gemv: out_dtype must be F16 or F32");
   FR_TRY(check_weight(w, 0, 0));
-  Gemv a;
-  a.x = (const h1*)x; a.w = to_wmat(w); a.y = y; a.out_f32 = out_dtype == FRHIP_F32;
-  const bool u8 = w->dtype == FRHIP_U8;
-  const int grid = decode_grid();
-  size_t lds = 2 * (size_t)w->K * (u8 ? 3 : 1);
-  FR_TRY(check_lds(lds));
-  const int R = pick_r(w->N, grid, u8);
-  DISPATCH_R_U8(gemv_kernel, R, u8, grid, lds, static_cast<hipStream_t>(s), a);
-  return check_launch("gemv");
+  RowsArgs a = empty_args(w->K);
+  a.prologue = P_COPY;
+  a.nvec = 1;
+  a.vec0 = (const h1*)x;
+  add_seg(a, w, 0, out_dtype == FRHIP_F32 ? E_STORE_F32 : E_STORE_F16, y);
+  return launch_rows(a, w->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "gemv");
 }

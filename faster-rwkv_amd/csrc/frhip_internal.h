@@ -14,7 +14,8 @@ int hip_result(hipError_t e, const char* what);
 // hipGetLastError() after a launch.
 int check_launch(const char* kernel);
 // Workgroups per launch for the row-streaming kernels: compute units of the
-// current device times FRHIP_WGS_PER_CU (default 2).
+// current device times FRHIP_WGS_PER_CU (default 1: with one 512-thread
+// workgroup per CU most decode launches are a single register-resident batch per wave).
 int decode_grid();
 int compute_units();
 

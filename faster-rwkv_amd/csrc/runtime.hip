@@ -12,7 +12,7 @@ namespace frhip {
 
 static thread_local std::string g_err = "no error";
 static int g_cus = 0;
-static int g_wgs_per_cu = 2;
+static int g_wgs_per_cu = 1;
 
 int set_error(int code, const char* msg) {
   g_err = msg ? msg : "error";
