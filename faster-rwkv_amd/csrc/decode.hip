@@ -467,6 +467,71 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   }
 }
 
+// ===========================================================================
+// RWKV-5.1/5.2 one-token state update, per head (kernels/cuda/att.cu:64-81,296-329):
+//   a_ij = k_i v_j ; tmp_ij = u_i a_ij + s_ij ; out_j = sum_i r_i tmp_ij ; s_ij <- w_i s_ij + a_ij
+// with the products and sums of tmp and s rounded separately (the reference uses
+// __fmul_rn/__fadd_rn there), then groupnorm over the head's S outputs (fp32, eps 1e-5),
+// rounding to half and the gate multiply in half.
+// One workgroup of 256 threads per head: thread t owns value index j = t % 64 and the
+// key rows i = (t / 64) * 16 ... +15; the four partial sums of out_j meet in LDS.
+// S must be 64.
+// ===========================================================================
+struct Wkv5One {
+  int H;
+  const float *s, *r, *k, *v, *w, *u, *lx_w, *lx_b;
+  const h1* g;
+  float* s_out;
+  h1* gated_out;
+};
+
+__global__ __launch_bounds__(256) void wkv5_one_kernel(Wkv5One a) {
+  constexpr int S = 64;
+  __shared__ float rk[3][S];      // r, k, v of this head
+  __shared__ float uw[2][S];      // u, w
+  __shared__ float part[4][S];
+  const int h = blockIdx.x, t = threadIdx.x;
+  const int j = t & 63, ig = t >> 6;
+  if (t < S) {
+    rk[0][t] = a.r[h * S + t];
+    rk[1][t] = a.k[h * S + t];
+    rk[2][t] = a.v[h * S + t];
+    uw[0][t] = a.u[h * S + t];
+    uw[1][t] = a.w[h * S + t];
+  }
+  const float* sh = a.s + (size_t)h * S * S;
+  float* so = a.s_out + (size_t)h * S * S;
+  float sreg[16];
+#pragma unroll
+  for (int ii = 0; ii < 16; ii++) sreg[ii] = sh[(ig * 16 + ii) * S + j];
+  __syncthreads();
+  const float vj = rk[2][j];
+  float acc = 0.f;
+#pragma unroll
+  for (int ii = 0; ii < 16; ii++) {
+    const int i = ig * 16 + ii;
+    const float aij = rk[1][i] * vj;
+    const float ua = uw[0][i] * aij;
+    const float tmp = ua + sreg[ii];
+    const float ws = uw[1][i] * sreg[ii];
+    so[i * S + j] = ws + aij;
+    acc += rk[0][i] * tmp;
+  }
+  part[ig][j] = acc;
+  __syncthreads();
+  if (t < S) {
+    const float o = ((part[0][t] + part[1][t]) + part[2][t]) + part[3][t];
+    const float mean = wave_sum(o) / (float)S;
+    const float d = o - mean;
+    float var = wave_sum(d * d) / (float)S;
+    var = var > 0.f ? var : 0.f;
+    const float inv = 1.0f / sqrtf(var + 1e-5f);
+    const int c = h * S + t;
+    const float y = d * inv * a.lx_w[c] + a.lx_b[c];
+    a.gated_out[c] = (h1)y * a.g[c];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -632,15 +697,17 @@ static void add_seg(RowsArgs& a, const frhip_weight* w, int vec, int epi, void* 
 using namespace frhip;
 
 extern "C" size_t frhip_decode_workspace_bytes(int C, int F) {
-  // rwkv [C] | r [C] | x_mid [C] | vx [F]   (binary16), each 256-byte aligned
+  // binary16 rwkv [C] | r [C] | x_mid [C] | g [C] ; fp32 k [C] | v [C] | r32 [C] ; binary16 vx [F];
+  // each 256-byte aligned (g, k, v, r32 serve RWKV-5 only)
   auto al = [](size_t n) { return (n + 255) / 256 * 256; };
   if (C <= 0 || F <= 0) return 0;
-  return al(2 * (size_t)C) * 3 + al(2 * (size_t)F);
+  return al(2 * (size_t)C) * 4 + al(2 * (size_t)F) + al(4 * (size_t)C) * 3;
 }
 
 namespace {
 struct Workspace {
-  h1 *rwkv, *r, *vx, *xmid;
+  h1 *rwkv, *r, *vx, *xmid, *g;
+  float *k32, *v32, *r32;
 };
 Workspace carve(void* ws, int C) {
   auto al = [](size_t n) { return (n + 255) / 256 * 256; };
@@ -652,6 +719,14 @@ Workspace carve(void* ws, int C) {
   p += al(2 * (size_t)C);
   w.xmid = reinterpret_cast<h1*>(p);
   p += al(2 * (size_t)C);
+  w.g = reinterpret_cast<h1*>(p);
+  p += al(2 * (size_t)C);
+  w.k32 = reinterpret_cast<float*>(p);
+  p += al(4 * (size_t)C);
+  w.v32 = reinterpret_cast<float*>(p);
+  p += al(4 * (size_t)C);
+  w.r32 = reinterpret_cast<float*>(p);
+  p += al(4 * (size_t)C);
   w.vx = reinterpret_cast<h1*>(p);
   return w;
 }
@@ -720,6 +795,66 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   b.res_x = (const h1*)x;
   add_seg(b, ow, 0, E_RESIDUAL, x_out);
   return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_out");
+}
+
+extern "C" int frhip_att_one_v5_1(int C, int H, const void* x, const void* sx, const float* s, const void* ln_w,
+                                  const void* ln_b, const float* lx_w, const float* lx_b, const void* k_mix,
+                                  const void* v_mix, const void* r_mix, const void* g_mix, const float* t_decay,
+                                  const float* t_first, const frhip_weight* kw, const frhip_weight* vw,
+                                  const frhip_weight* rw, const frhip_weight* gw, const frhip_weight* ow,
+                                  void* x_out, void* xx_out, float* s_out, void* workspace, frhip_stream s_) {
+  FR_TRY(check_embd(C));
+  if (H <= 0 || C % H != 0 || C / H != 64) return set_error(FRHIP_ESHAPE, "att_one_v5_1: head size must be 64");
+  FR_TRY(check_vec(x, "x is null or misaligned"));
+  FR_TRY(check_vec(sx, "sx is null or misaligned"));
+  FR_TRY(check_vec(ln_w, "ln_w is null or misaligned"));
+  FR_TRY(check_vec(ln_b, "ln_b is null or misaligned"));
+  FR_TRY(check_vec(k_mix, "k_mix is null or misaligned"));
+  FR_TRY(check_vec(v_mix, "v_mix is null or misaligned"));
+  FR_TRY(check_vec(r_mix, "r_mix is null or misaligned"));
+  FR_TRY(check_vec(g_mix, "g_mix is null or misaligned"));
+  FR_TRY(check_vec(x_out, "x_out is null or misaligned"));
+  FR_TRY(check_vec(xx_out, "xx_out is null or misaligned"));
+  FR_TRY(check_vec(workspace, "workspace is null or misaligned"));
+  if (!s || !s_out || !lx_w || !lx_b || !t_decay || !t_first) return set_error(FRHIP_EINVAL, "att_one_v5_1: null state or parameter");
+  if (xx_out == sx) return set_error(FRHIP_EINVAL, "att_one_v5_1: xx_out must not alias sx");
+  FR_TRY(check_weight(kw, C, C));
+  FR_TRY(check_weight(vw, C, C));
+  FR_TRY(check_weight(rw, C, C));
+  FR_TRY(check_weight(gw, C, C));
+  FR_TRY(check_weight(ow, C, C));
+  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype || kw->dtype != gw->dtype)
+    return set_error(FRHIP_EINVAL, "att_one_v5_1: key/value/receptance/gate dtypes differ");
+  hipStream_t st = static_cast<hipStream_t>(s_);
+  Workspace w = carve(workspace, C);
+
+  // LN -> 4 mixes -> k, v, r (fp32) and g = silu(.) (half)      att.cu:276-290
+  RowsArgs a = empty_args(C);
+  a.prologue = P_LN_MIX;
+  a.nvec = 4;
+  a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+  a.mix[0] = (const h1*)k_mix; a.mix[1] = (const h1*)v_mix; a.mix[2] = (const h1*)r_mix; a.mix[3] = (const h1*)g_mix;
+  a.xx_out = (h1*)xx_out;
+  add_seg(a, kw, 0, E_STORE_F32, w.k32);
+  add_seg(a, vw, 1, E_STORE_F32, w.v32);
+  add_seg(a, rw, 2, E_STORE_F32, w.r32);
+  add_seg(a, gw, 3, E_SILU, w.g);
+  FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "att_v5_front"));
+
+  Wkv5One k;
+  k.H = H;
+  k.s = s; k.r = w.r32; k.k = w.k32; k.v = w.v32; k.w = t_decay; k.u = t_first; k.lx_w = lx_w; k.lx_b = lx_b;
+  k.g = w.g; k.s_out = s_out; k.gated_out = w.rwkv;
+  hipLaunchKernelGGL(wkv5_one_kernel, dim3(H), dim3(256), 0, st, k);
+  FR_TRY(check_launch("wkv5_one"));
+
+  RowsArgs b = empty_args(C);
+  b.prologue = P_COPY;
+  b.nvec = 1;
+  b.vec0 = w.rwkv;
+  b.res_x = (const h1*)x;
+  add_seg(b, ow, 0, E_RESIDUAL, x_out);
+  return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_v5_out");
 }
 
 extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const void* ln_w, const void* ln_b,

@@ -32,9 +32,12 @@ struct DecodePlan {
   float *logits_host[2] = {nullptr, nullptr};  // pinned; the graph's last node copies into it
   int32_t *ring = nullptr;                     // pinned; token ids, read by the first kernel
   uint32_t fed = 0;                            // tokens fed so far == the device counter
-  std::vector<Tensor> aa, bb, pp;
+  bool v5 = false;                      // RWKV-5.1/5.2: state is (shift, [H,S,S] matrix, shift)
+  int H = 0;
+  std::vector<Tensor> aa, bb, pp;       // RWKV-4
+  std::vector<Tensor> wkv;              // RWKV-5
   std::vector<Tensor> sx_att[2], sx_ffn[2];
-  std::vector<std::vector<Tensor>> views[2];  // views[parity][layer] = the 5 state tensors model code sees
+  std::vector<std::vector<Tensor>> views[2];  // views[parity][layer] = the state tensors model code sees
   int parity = 0;                             // which ping-pong side holds the current shift states
   frhip_graph graph[2] = {nullptr, nullptr};
   bool use_graph = true;
@@ -51,6 +54,8 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   auto p = std::make_shared<DecodePlan>();
   p->L = model->n_layer();
   p->C = model->n_embd();
+  p->v5 = model->version() != "4";
+  p->H = model->head_size();
   p->F = model->n_ffn() > 0 ? model->n_ffn() : static_cast<int>(model->_params[15].size(1));
   p->V = static_cast<int>(ex.emb_table.size(0));
   const int C = p->C;
@@ -69,9 +74,13 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
     lh = static_cast<float *>(h);
   }
   for (int l = 0; l < p->L; l++) {
-    p->aa.push_back(Tensor::Empty({C}, DType::kFloat32, d));
-    p->bb.push_back(Tensor::Empty({C}, DType::kFloat32, d));
-    p->pp.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+    if (p->v5) {
+      p->wkv.push_back(Tensor::Empty({p->H, C / p->H, C / p->H}, DType::kFloat32, d));
+    } else {
+      p->aa.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+      p->bb.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+      p->pp.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+    }
     for (int s = 0; s < 2; s++) {
       p->sx_att[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
       p->sx_ffn[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
@@ -79,8 +88,12 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   }
   for (int s = 0; s < 2; s++) {
     p->views[s].resize(p->L);
-    for (int l = 0; l < p->L; l++)
-      p->views[s][l] = {p->sx_att[s][l], p->aa[l], p->bb[l], p->pp[l], p->sx_ffn[s][l]};
+    for (int l = 0; l < p->L; l++) {
+      if (p->v5)
+        p->views[s][l] = {p->sx_att[s][l], p->wkv[l], p->sx_ffn[s][l]};
+      else
+        p->views[s][l] = {p->sx_att[s][l], p->aa[l], p->bb[l], p->pp[l], p->sx_ffn[s][l]};
+    }
   }
   p->use_graph = std::getenv("FR_HIP_NO_GRAPH") == nullptr;  // fixed when the model first runs
   return p;
@@ -92,9 +105,9 @@ static void adopt_states(Model *model, DecodePlan &p) {
   auto &st = model->states();
   RV_CHECK(static_cast<int>(st.size()) == p.L);
   for (int l = 0; l < p.L; l++) {
-    RV_CHECK(st[l].size() == 5);
     auto &mine = p.views[p.parity][l];
-    for (int j = 0; j < 5; j++) {
+    RV_CHECK(st[l].size() == mine.size());
+    for (size_t j = 0; j < mine.size(); j++) {
       if (st[l][j].data_ptr() == mine[j].data_ptr()) continue;
       RV_CHECK(st[l][j].nbytes() == mine[j].nbytes() && st[l][j].dtype() == mine[j].dtype())
           << "state " << l << "/" << j << " has the wrong shape or dtype";
@@ -114,7 +127,26 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
   FRHIP_CHECK(frhip_embed_ring(ex.emb_table.data_ptr(), p.V, 2 * C, p.ring, DecodePlan::kRing,
                                reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
   size_t pi = 0;
-  for (int l = 0; l < p.L; l++) {
+  for (int l = 0; l < p.L && p.v5; l++) {
+    const frhip_weight *kw = find_weight(P[pi + 10]), *vw = find_weight(P[pi + 11]), *rw = find_weight(P[pi + 12]),
+                       *gw = find_weight(P[pi + 13]), *ow = find_weight(P[pi + 14]);
+    RV_CHECK(kw && vw && rw && gw && ow);
+    FRHIP_CHECK(frhip_att_one_v5_1(C, p.H, p.x.data_ptr(), p.sx_att[cur][l].data_ptr(), p.wkv[l].data_ptr<float>(),
+                                   P[pi].data_ptr(), P[pi + 1].data_ptr(), P[pi + 2].data_ptr<float>(),
+                                   P[pi + 3].data_ptr<float>(), P[pi + 4].data_ptr(), P[pi + 5].data_ptr(),
+                                   P[pi + 6].data_ptr(), P[pi + 7].data_ptr(), P[pi + 8].data_ptr<float>(),
+                                   P[pi + 9].data_ptr<float>(), kw, vw, rw, gw, ow, p.x.data_ptr(),
+                                   p.sx_att[nxt][l].data_ptr(), p.wkv[l].data_ptr<float>(), p.ws.data_ptr(), s));
+    pi += 15;
+    const frhip_weight *fk = find_weight(P[pi + 4]), *fv = find_weight(P[pi + 5]), *frw = find_weight(P[pi + 6]);
+    RV_CHECK(fk && fv && frw);
+    FRHIP_CHECK(frhip_ffn_one(C, F, p.x.data_ptr(), p.sx_ffn[cur][l].data_ptr(), P[pi].data_ptr(),
+                              P[pi + 1].data_ptr(), P[pi + 2].data_ptr(), P[pi + 3].data_ptr(), fk, fv, frw,
+                              p.x.data_ptr(), p.sx_ffn[nxt][l].data_ptr(), (l + 1) % 6 == 0 ? 1 : 0, p.ws.data_ptr(),
+                              s));
+    pi += 7;
+  }
+  for (int l = 0; l < p.L && !p.v5; l++) {
     const frhip_weight *kw = find_weight(P[pi + 7]), *vw = find_weight(P[pi + 8]), *rw = find_weight(P[pi + 9]),
                        *ow = find_weight(P[pi + 10]);
     RV_CHECK(kw && vw && rw && ow);
@@ -143,7 +175,8 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
 
 Tensor ModelForward(Model *model, Device device, int id) {
   const bool generic = std::getenv("FR_HIP_GENERIC") != nullptr;  // read per call so that one process can compare both paths
-  if (generic || model->version() != "4") return def::ModelForward(model, device, id);
+  const std::string &ver = model->version();
+  if (generic || !(ver == "4" || ver == "5.1" || ver == "5.2")) return def::ModelForward(model, device, id);
   auto ex = extra_of(model);
   if (!ex->plan) ex->plan = make_plan(model, *ex);
   DecodePlan &p = *ex->plan;
@@ -173,9 +206,10 @@ Tensor ModelForward(Model *model, Device device, int id) {
   p.fed++;  // the device counter advances when the first kernel of the step runs
   p.parity = 1 - cur;
   auto &st = model->states();
+  const size_t last = p.v5 ? 2 : 4;
   for (int l = 0; l < p.L; l++) {
     st[l][0] = p.views[p.parity][l][0];
-    st[l][4] = p.views[p.parity][l][4];
+    st[l][last] = p.views[p.parity][l][last];
   }
   // The graph's last node has copied the logits into pinned host memory; waiting for the stream
   // is the step's one synchronisation point (the reference's is the blocking cudaMemcpy in

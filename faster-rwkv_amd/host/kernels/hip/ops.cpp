@@ -161,6 +161,31 @@ std::tuple<Tensor, Tensor> ffn(const Tensor &x, const Tensor &sx, const Tensor &
   return {x_out, xx};
 }
 
+// att_one_v5_1, RWKV-5.1/5.2 one token (reference: kernels/cuda/att.cu:393-425).
+std::tuple<Tensor, Tensor, Tensor>
+att_one_v5_1(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &ln_w, const Tensor &ln_b,
+             const Tensor &lx_w, const Tensor &lx_b, const Tensor &k_mix, const Tensor &v_mix, const Tensor &r_mix,
+             const Tensor &g_mix, const Tensor &t_decay, const Tensor &t_first, const Tensor &kw, const Tensor &vw,
+             const Tensor &rw, const Tensor &gw, const Tensor &ow) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 1);
+  const int C = static_cast<int>(x.size(0));
+  const int H = static_cast<int>(t_decay.size(0));
+  frhip_weight d[5];
+  Tensor tmp[5];
+  const frhip_weight *w[5] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
+                              weight_of(gw, d[3], tmp[3]), weight_of(ow, d[4], tmp[4])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor s_out = Tensor::Empty(s.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor ws = workspace(C, 16);
+  FRHIP_CHECK(frhip_att_one_v5_1(C, H, x.data_ptr(), sx.data_ptr(), s.data_ptr<float>(), ln_w.data_ptr(),
+                                 ln_b.data_ptr(), lx_w.data_ptr<float>(), lx_b.data_ptr<float>(), k_mix.data_ptr(),
+                                 v_mix.data_ptr(), r_mix.data_ptr(), g_mix.data_ptr(), t_decay.data_ptr<float>(),
+                                 t_first.data_ptr<float>(), w[0], w[1], w[2], w[3], w[4], x_out.data_ptr(),
+                                 xx.data_ptr(), s_out.data_ptr<float>(), ws.data_ptr(), stream()));
+  return {x_out, xx, s_out};
+}
+
 KernelRegister fill_reg("fill_", Device::kHIP, fill_);
 KernelRegister cast_reg("cast_dtype", Device::kHIP, cast_dtype);
 KernelRegister scalar_div_reg("scalar_div_", Device::kHIP, scalar_div_);
@@ -170,6 +195,7 @@ KernelRegister matmul_reg("matmul", Device::kHIP, matmul);
 KernelRegister vgather_reg("vgather", Device::kHIP, vgather);
 KernelRegister att_reg("att", Device::kHIP, att);
 KernelRegister ffn_reg("ffn", Device::kHIP, ffn);
+KernelRegister att_one_v5_1_reg("att_one_v5_1", Device::kHIP, att_one_v5_1);
 
 }  // namespace hip
 }  // namespace rwkv

@@ -89,11 +89,12 @@ def test_ffn_one(C_, F_, quant, div2):
     # the last product by one spacing, so the end-to-end comparison is loose ...
     assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
     # ... and the strict one restarts the oracle from the kernel's own intermediates
-    # (workspace: rwkv | r | x_mid | vx, each rounded up to 256 bytes): bit-exact.
+    # (workspace: binary16 rwkv | r | x_mid | g, fp32 k | v | r32, binary16 vx; each rounded up
+    # to 256 bytes): bit-exact.
     ws = wsb.numpy()
     al = lambda n: (n + 255) // 256 * 256
     r_g = ws[al(2 * C_) // 2:][:C_]
-    vx_g = ws[3 * al(2 * C_) // 2:][:F_]
+    vx_g = ws[(4 * al(2 * C_) + 3 * al(4 * C_)) // 2:][:F_]
     r_ref = po.sigmoid_f16(po.gemm_f16(po.mix_f16(ref_xx, sx, mr), rref, "f16"))
     vx_ref = po.relu_square_f16(po.gemm_f16(po.mix_f16(ref_xx, sx, mk), kref, "f16"))
     assert_close_f16(r_g, r_ref, max_ulp=1, max_frac=0.01, what="r")
@@ -104,6 +105,39 @@ def test_ffn_one(C_, F_, quant, div2):
     if div2:
         strict = (strict.astype(np.float32) / 2).astype(np.float16)
     assert_close_f16(x_out.numpy(), strict, max_ulp=1, max_frac=0.002, what="x_out from kernel intermediates")
+
+
+@pytest.mark.parametrize("C_,H_", [(2560, 40), (512, 8)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_att_one_v5_1(C_, H_, quant):
+    """kernels/cuda/att.cu:267-335,393-425 (serves RWKV-5.1 and 5.2)."""
+    S_ = C_ // H_
+    x, sx = h(rng.standard_normal(C_) * 2), h(rng.standard_normal(C_))
+    s = rng.standard_normal((H_, S_, S_)).astype(np.float32)
+    ln_w, ln_b = h(1 + 0.1 * rng.standard_normal(C_)), h(0.1 * rng.standard_normal(C_))
+    lx_w = (1 + 0.1 * rng.standard_normal(C_)).astype(np.float32)
+    lx_b = (0.1 * rng.standard_normal(C_)).astype(np.float32)
+    mixes = [h(rng.uniform(0, 1, C_)) for _ in range(4)]
+    td = np.exp(-np.exp(rng.uniform(-6, 0, (H_, S_)))).astype(np.float32)
+    tf = rng.uniform(-1, 1, (H_, S_)).astype(np.float32)
+    ws, refs = [], []
+    for _ in range(5):
+        w, r = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+        ws.append(w)
+        refs.append(r)
+    ref_x, ref_xx, ref_s = po.att_v5_2_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, *mixes, td, tf, *refs, H_)
+    x_out, xx_out = DevBuf.empty(C_, np.float16), DevBuf.empty(C_, np.float16)
+    s_out = DevBuf.empty((H_, S_, S_), np.float32)
+    wsb = DevBuf(L().frhip_decode_workspace_bytes(C_, 4 * C_))
+    fr.check(L().frhip_att_one_v5_1(C_, H_, keep(x).ptr, keep(sx).ptr, keep(s).ptr, keep(ln_w).ptr, keep(ln_b).ptr,
+                                    keep(lx_w).ptr, keep(lx_b).ptr, *[keep(m).ptr for m in mixes], keep(td).ptr,
+                                    keep(tf).ptr, *[w.ref for w in ws], x_out.ptr, xx_out.ptr, s_out.ptr, wsb.ptr,
+                                    None))
+    assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx")
+    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-5, atol=1e-5)
+    # groupnorm amplifies the fp32 summation-order noise of the head outputs; a few one-spacing
+    # flips of the gated vector then spread over the output product
+    assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
 
 
 @pytest.mark.parametrize("quant", [False, True])

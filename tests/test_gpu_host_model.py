@@ -122,3 +122,31 @@ def test_bad_arguments_surface_as_exceptions(model_files):
     with pytest.raises(fr.FrhipError):
         m.run(V_ + 5)
     m.close()
+
+
+def test_rwkv5_2_model_matches_oracle(tmp_path):
+    """RWKV-5.2 (config-5 architecture at reduced size): fused graph path through Model::Run."""
+    L5, C5, F5, V5, H5 = 6, 512, 1792, 2048, 8
+    params, emb = make_model(52, L5, C5, F5, V5, H5, seed=21)
+    path = str(tmp_path / "v52.fr")
+    fr.write_fr(path, "5.2", L5, C5, F5, H5, params, emb)
+    for strategy in ("hip fp16", "hip int8"):
+        p = list(params)
+        if strategy.endswith("int8"):
+            for i in matrix_indices(52, L5):
+                p[i] = po.dequant_u8(*quantize_u8(params[i]))
+        om = po.Model(52, po.F16, L5, C5, F5, H5, V5, p, emb)
+        m = fr.Model(path, strategy)
+        assert m.n_head == H5 and m.n_ffn == F5
+        tok, worst = 11, 0.0
+        for step in range(64):
+            lh, lo = m.run(tok), om.run(tok)
+            worst = max(worst, float(np.abs(lh - lo).max()))
+            assert int(np.argmax(lh)) == int(np.argmax(lo)), "greedy token differs at step %d" % step
+            tok = int(np.argmax(lo))
+        print(strategy, "v5.2 worst |dlogit| over 64 steps:", worst, flush=True)
+        assert worst <= 2e-2
+        s_ref = om.state[5 * 3 + 1]
+        s_got = m.state(5, 1, np.float32)
+        assert np.abs(s_got - s_ref).max() <= 5e-3 * np.abs(s_ref).max()
+        m.close()
