@@ -1,0 +1,41 @@
+// Argument structures of the MFMA GEMM shared by gemm.hip and seq.hip.
+#pragma once
+
+#include "device_utils.h"
+#include "frhip_internal.h"
+
+namespace frhip {
+
+constexpr int kGemmMaxSeg = 4;
+
+enum GemmEpi : int {
+  G_STORE_F16 = 0,
+  G_STORE_F32 = 1,
+  G_SIGMOID = 2,    // half(sigmoid(half(acc)))                        ffn_seq.cu:78-79, att.cu:203
+  G_RELU2 = 3,      // relu(half(acc))^2                               ffn_seq.cu:80-81
+  G_SILU = 4,       // silu(half(acc))                                 att_seq.cu:394-395
+  G_RESIDUAL = 5,   // x + half(acc)                                   att_seq.cu:412-415
+  G_FFN_OUT = 6     // fma(half(acc), r, x) [/ 2]                      ffn_seq.cu:82-85, model_forward_seq.cpp:163-165
+};
+
+struct GemmSeg {
+  const h1* A;                       // [M][K]
+  const unsigned char* B;            // [N][K] binary16 or uint8
+  const h1 *mx, *rx, *my, *ry;       // uint8 only
+  void* out;                         // [M][N]
+  int N, epi;
+};
+
+struct GemmArgs {
+  int M, K, nseg;
+  int tile_start[kGemmMaxSeg + 1];  // first N-tile of each segment
+  GemmSeg seg[kGemmMaxSeg];
+  const h1* res_x;  // [M][N] G_RESIDUAL, G_FFN_OUT
+  const h1* res_r;  // [M][N] G_FFN_OUT
+  int div2;
+};
+
+int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what);
+void gemm_add_seg(GemmArgs& a, const void* A, const frhip_weight* w, void* out, int epi);
+
+}  // namespace frhip

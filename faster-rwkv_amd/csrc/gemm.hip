@@ -1,0 +1,235 @@
+// Seq-mode (prefill) matrix products on the MFMA units of gfx950.
+//
+//   Y[T, N] = X[T, K] . W        with W held output-major, Wt[N][K]
+//
+// Both operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
+// a lane's A (or B) fragment is 8 consecutive k of one row, i.e. one 16-byte load.
+// Workgroup tile 128x128, K step 64, 256 threads = 2x2 waves of 64x64 (2x2 MFMA tiles,
+// 64 fp32 accumulators per lane).  Tiles of X and Wt go global -> registers -> LDS
+// (rows padded by 16 bytes against bank conflicts); the loads of step k+1 are issued
+// before the MFMAs of step k.  uint8 weights are dequantised to binary16 on their way
+// into LDS with the same formula as the one-token kernels, so the product sees exactly
+// the dequantised matrix.  Products are exact in fp32, accumulation is fp32, and the
+// result is rounded once to the output type (kernels/cuda/matmul.cpp:38-42,64-68).
+// Independent products over the same T and K share one launch ("segments"), each with
+// its own X, W and fused epilogue.
+#include <climits>
+#include <cstring>
+
+#include "gemm.h"
+
+#pragma clang fp contract(off)
+
+namespace frhip {
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 64, LDSK = BK + 8;
+constexpr int kGemmThreads = 256;
+template <bool U8>
+__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
+  __shared__ __attribute__((aligned(16))) h1 As[BM][LDSK];
+  __shared__ __attribute__((aligned(16))) h1 Bs[BN][LDSK];
+
+  // which segment does this N-tile belong to
+  int sidx = 0;
+#pragma unroll
+  for (int i = 1; i < kGemmMaxSeg; i++) sidx += (i < a.nseg && (int)blockIdx.x >= a.tile_start[i]) ? 1 : 0;
+  const GemmSeg& sg = a.seg[sidx];
+  const int n0 = ((int)blockIdx.x - a.tile_start[sidx]) * BN;
+  const int m0 = blockIdx.y * BM;
+  const int M = a.M, K = a.K, N = sg.N;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // global -> register staging: a tile is 128 rows x 64 k.
+  //   A (binary16): 1024 chunks of 8 halves, 4 per thread: chunk c -> row c/8, k (c%8)*8
+  //   B binary16: same.  B uint8: 512 chunks of 16 codes, 2 per thread: row c/4, k (c%4)*16
+  h8 ra[4];
+  h8 rb[4];
+  u32x4 rq[2];
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int c = tid + i * kGemmThreads;
+      int row = m0 + (c >> 3);
+      row = row < M ? row : M - 1;  // rows past M are computed on a copy of the last row and never stored
+      ra[i] = *reinterpret_cast<const h8*>(sg.A + (size_t)row * K + k0 + (c & 7) * 8);
+    }
+    if constexpr (!U8) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int c = tid + i * kGemmThreads;
+        int row = n0 + (c >> 3);
+        row = row < N ? row : N - 1;
+        rb[i] = __builtin_nontemporal_load(reinterpret_cast<const h8*>(sg.B + ((size_t)row * K + k0 + (c & 7) * 8) * 2));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int c = tid + i * kGemmThreads;
+        int row = n0 + (c >> 2);
+        row = row < N ? row : N - 1;
+        rq[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sg.B + (size_t)row * K + k0 + (c & 3) * 16));
+      }
+    }
+  };
+  auto store_tiles = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int c = tid + i * kGemmThreads;
+      *reinterpret_cast<h8*>(&As[c >> 3][(c & 7) * 8]) = ra[i];
+    }
+    if constexpr (!U8) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int c = tid + i * kGemmThreads;
+        *reinterpret_cast<h8*>(&Bs[c >> 3][(c & 7) * 8]) = rb[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int c = tid + i * kGemmThreads;
+        int row = n0 + (c >> 2);
+        row = row < N ? row : N - 1;
+        const int kk = k0 + (c & 3) * 16;
+        const h1 c255 = dequant_c255(sg.rx[row]);
+        const h2 c2 = {c255, c255};
+        const h1 mxv = sg.mx[row];
+        const h2 m2 = {mxv, mxv};
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+          const h8 ry = *reinterpret_cast<const h8*>(sg.ry + kk + hh * 8);
+          const h8 my = *reinterpret_cast<const h8*>(sg.my + kk + hh * 8);
+          const uint32_t w0 = rq[i][2 * hh], w1 = rq[i][2 * hh + 1];
+          h2 p0 = dequant_pair<0>(w0, c2, m2, ry.s01, my.s01);
+          h2 p1 = dequant_pair<1>(w0, c2, m2, ry.s23, my.s23);
+          h2 p2 = dequant_pair<0>(w1, c2, m2, ry.s45, my.s45);
+          h2 p3 = dequant_pair<1>(w1, c2, m2, ry.s67, my.s67);
+          h8 o = {p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+          *reinterpret_cast<h8*>(&Bs[c >> 2][(c & 3) * 16 + hh * 8]) = o;
+        }
+      }
+    }
+  };
+
+  f16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  load_tiles(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();  // everyone is done reading the previous tile
+    store_tiles(k0);
+    __syncthreads();
+    if (k0 + BK < K) load_tiles(k0 + BK);
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      h8 fa[2], fb[2];
+      const int kofs = ks + (lane >> 5) * 8;
+#pragma unroll
+      for (int i = 0; i < 2; i++) fa[i] = *reinterpret_cast<const h8*>(&As[wm * 64 + i * 32 + (lane & 31)][kofs]);
+#pragma unroll
+      for (int j = 0; j < 2; j++) fb[j] = *reinterpret_cast<const h8*>(&Bs[wn * 64 + j * 32 + (lane & 31)][kofs]);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // epilogue: acc[i][j][v] is C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the 32x32 tile
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (row < M && col < N) {
+          const float s = acc[i][j][v];
+          const size_t o = (size_t)row * N + col;
+          switch (sg.epi) {
+            case G_STORE_F16: static_cast<h1*>(sg.out)[o] = (h1)s; break;
+            case G_STORE_F32: static_cast<float*>(sg.out)[o] = s; break;
+            case G_SIGMOID: static_cast<h1*>(sg.out)[o] = sigmoid_h((h1)s); break;
+            case G_RELU2: {
+              const h1 t = (h1)s;
+              static_cast<h1*>(sg.out)[o] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
+              break;
+            }
+            case G_SILU: static_cast<h1*>(sg.out)[o] = silu_h((h1)s); break;
+            case G_RESIDUAL: static_cast<h1*>(sg.out)[o] = a.res_x[o] + (h1)s; break;
+            case G_FFN_OUT: {
+              h1 r = __builtin_fmaf16((h1)s, a.res_r[o], a.res_x[o]);
+              if (a.div2) r = r / (h1)2.0f;
+              static_cast<h1*>(sg.out)[o] = r;
+              break;
+            }
+            default: break;
+          }
+        }
+      }
+    }
+  }
+}
+
+int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what) {
+  if (a.M <= 0) return 0;
+  if (a.K <= 0 || a.K % BK != 0) return set_error(FRHIP_ESHAPE, "gemm: K must be a positive multiple of 64");
+  int tiles = 0;
+  for (int s = 0; s < a.nseg; s++) {
+    a.tile_start[s] = tiles;
+    tiles += (a.seg[s].N + BN - 1) / BN;
+  }
+  for (int s = a.nseg; s <= kGemmMaxSeg; s++) a.tile_start[s] = INT_MAX;
+  a.tile_start[a.nseg] = tiles;
+  dim3 grid(tiles, (a.M + BM - 1) / BM);
+  if (u8)
+    hipLaunchKernelGGL(gemm_kernel<true>, grid, dim3(kGemmThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL(gemm_kernel<false>, grid, dim3(kGemmThreads), 0, st, a);
+  return check_launch(what);
+}
+
+void gemm_add_seg(GemmArgs& a, const void* A, const frhip_weight* w, void* out, int epi) {
+  GemmSeg& s = a.seg[a.nseg++];
+  s.A = static_cast<const h1*>(A);
+  s.B = static_cast<const unsigned char*>(w->data);
+  s.mx = static_cast<const h1*>(w->mx);
+  s.rx = static_cast<const h1*>(w->rx);
+  s.my = static_cast<const h1*>(w->my);
+  s.ry = static_cast<const h1*>(w->ry);
+  s.out = out;
+  s.N = w->N;
+  s.epi = epi;
+}
+
+}  // namespace frhip
+
+using namespace frhip;
+
+// matmul, matrix x matrix (kernels/cuda/matmul.cpp:110-121): x [T][K] binary16, y [T][N].
+extern "C" int frhip_gemm(const void* x, const frhip_weight* w, void* y, int T, int out_dtype, frhip_stream s) {
+  if (!x || !w || !w->data || !y) return set_error(FRHIP_EINVAL, "gemm: null pointer");
+  if (T < 0) return set_error(FRHIP_ESHAPE, "gemm: negative T");
+  if (out_dtype != FRHIP_F16 && out_dtype != FRHIP_F32) return set_error(FRHIP_EINVAL, "gemm: out_dtype must be F16 or F32");
+  if (w->dtype != FRHIP_F16 && w->dtype != FRHIP_U8) return set_error(FRHIP_EINVAL, "gemm: weight dtype must be F16 or U8");
+  if (w->dtype == FRHIP_U8 && (!w->mx || !w->rx || !w->my || !w->ry)) return set_error(FRHIP_EINVAL, "gemm: uint8 weight without mx/rx/my/ry");
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(w->data) % 16 != 0)
+    return set_error(FRHIP_EINVAL, "gemm: operands must be 16-byte aligned");
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = T;
+  a.K = w->K;
+  gemm_add_seg(a, x, w, y, out_dtype == FRHIP_F32 ? G_STORE_F32 : G_STORE_F16);
+  return launch_gemm(a, w->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "gemm");
+}

@@ -1,0 +1,522 @@
+// Seq-mode (prompt) operators: layernorm + token shift + mix over T rows, the WKV scans of
+// RWKV-4 and RWKV-5.2, and the att_seq / ffn_seq compositions around the MFMA GEMM.
+//
+// Both recurrences are linear in their state, so the scans run CHUNKED over time instead of
+// as one serial loop of T steps on a handful of wavefronts (kernels/cuda/att_seq.cu:258-322
+// runs 64 threads per head for T steps):
+//   1. every chunk is scanned from an EMPTY state, all chunks in parallel -> local end states;
+//   2. a short serial pass over the chunks turns local end states into the true state at the
+//      start of every chunk (state_in[c+1] = decay^len(state_in[c]) + local[c]);
+//   3. every chunk is scanned again from its true start state, all chunks in parallel,
+//      producing the outputs; the last chunk leaves the final state.
+// The arithmetic of pass 3 is the one-token recurrence (kernels/cuda/att.cu:30-62, :64-81);
+// only the representation of the carried state differs from a serial scan, at fp32 rounding level.
+#include <climits>
+#include <cstring>
+
+#include "gemm.h"
+
+#pragma clang fp contract(off)
+
+namespace frhip {
+
+// ---------------------------------------------------------------------------
+// layernorm + token shift + mix for T rows: one workgroup (256 threads) per row.
+//   xx_t = LN(x_t) ; sx_t = (t == 0) ? state : xx_{t-1} ; out_i[t] = mix(xx_t, sx_t, mix_i)
+// (kernels/cuda/ffn_seq.cu:70-77, att_seq.cu:379-389).  LN(x_{t-1}) is recomputed by the
+// workgroup of row t, which saves a [T, C] round trip.  Row T-1 also writes xx_{T-1}, the
+// new shift state.
+// ---------------------------------------------------------------------------
+struct LnMixSeq {
+  int T, C, nmix;
+  const h1 *x, *state, *ln_w, *ln_b;
+  const h1* mix[4];
+  h1* out[4];
+  h1* xx_last;
+};
+
+__device__ __forceinline__ void ln_row_to_lds(const h1* xr, const h1* g, const h1* b, int C, h1* dst, float* red) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < C; i += 256) s += (float)xr[i];
+  const float mean = block_sum<4>(s, red) / (float)C;
+  float q = 0.f;
+  for (int i = threadIdx.x; i < C; i += 256) {
+    float d = (float)xr[i] - mean;
+    q += d * d;
+  }
+  float var = block_sum<4>(q, red) / (float)C;
+  var = var > 0.f ? var : 0.f;
+  const float inv = 1.0f / sqrtf(var + 1e-5f);
+  for (int i = threadIdx.x; i < C; i += 256) {
+    h1 n = (h1)(((float)xr[i] - mean) * inv);
+    dst[i] = (n * g[i]) + b[i];
+  }
+}
+
+__global__ __launch_bounds__(256) void ln_mix_seq_kernel(LnMixSeq a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ float red[4];
+  h1* cur = reinterpret_cast<h1*>(smem);
+  h1* prev = cur + a.C;
+  const int t = blockIdx.x, C = a.C;
+  ln_row_to_lds(a.x + (size_t)t * C, a.ln_w, a.ln_b, C, cur, red);
+  if (t == 0) {
+    for (int i = threadIdx.x; i < C; i += 256) prev[i] = a.state[i];
+  } else {
+    ln_row_to_lds(a.x + (size_t)(t - 1) * C, a.ln_w, a.ln_b, C, prev, red);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < C; i += 256) {
+    const h1 xx = cur[i], sx = prev[i];
+    for (int m = 0; m < a.nmix; m++) a.out[m][(size_t)t * C + i] = mix1(xx, sx, a.mix[m][i]);
+    if (t == a.T - 1) a.xx_last[i] = xx;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// RWKV-4 WKV scan.  k, v [T][C] fp32; r [T][C] half (already through the sigmoid),
+// overwritten with r * half(wkv).
+// ---------------------------------------------------------------------------
+struct Wkv4Seq {
+  int T, C, Lc, nchunk;
+  const float *k, *v, *u, *w;
+  h1* r;
+  const float *aa, *bb, *pp;  // state before the sequence
+  float *la, *lb, *lp;        // [nchunk][C] local end states (pass 1)
+  float *sa, *sb, *sp;        // [nchunk][C] state at the start of each chunk (pass 2)
+  float *aa_out, *bb_out, *pp_out;
+};
+
+__global__ __launch_bounds__(256) void wkv4_local_kernel(Wkv4Seq a) {
+  const int c = blockIdx.x * 256 + threadIdx.x, ch = blockIdx.y;
+  if (c >= a.C) return;
+  const int t0 = ch * a.Lc, t1 = min(t0 + a.Lc, a.T);
+  const float w = a.w[c];
+  float aa = 0.f, bb = 0.f, pp = -1e30f;
+  for (int t = t0; t < t1; t++) {
+    const float k = a.k[(size_t)t * a.C + c], v = a.v[(size_t)t * a.C + c];
+    const float ww = w + pp;
+    const float p = (ww > k) ? ww : k;
+    const float e1 = expf(ww - p), e2 = expf(k - p);
+    aa = e1 * aa + e2 * v;
+    bb = e1 * bb + e2;
+    pp = p;
+  }
+  const size_t o = (size_t)ch * a.C + c;
+  a.la[o] = aa;
+  a.lb[o] = bb;
+  a.lp[o] = pp;
+}
+
+__global__ __launch_bounds__(256) void wkv4_carry_kernel(Wkv4Seq a) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= a.C) return;
+  const float w = a.w[c];
+  float aa = a.aa[c], bb = a.bb[c], pp = a.pp[c];
+  for (int ch = 0; ch < a.nchunk; ch++) {
+    const size_t o = (size_t)ch * a.C + c;
+    a.sa[o] = aa;
+    a.sb[o] = bb;
+    a.sp[o] = pp;
+    const int len = min(a.Lc, a.T - ch * a.Lc);
+    // the incoming state decays by len steps; the chunk's own tokens contribute its local state
+    const float pd = pp + (float)len * w;
+    const float lp = a.lp[o];
+    const float p = (pd > lp) ? pd : lp;
+    const float e1 = expf(pd - p), e2 = expf(lp - p);
+    aa = e1 * aa + e2 * a.la[o];
+    bb = e1 * bb + e2 * a.lb[o];
+    pp = p;
+  }
+}
+
+__global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
+  const int c = blockIdx.x * 256 + threadIdx.x, ch = blockIdx.y;
+  if (c >= a.C) return;
+  const int t0 = ch * a.Lc, t1 = min(t0 + a.Lc, a.T);
+  const float w = a.w[c], u = a.u[c];
+  const size_t o = (size_t)ch * a.C + c;
+  float aa = a.sa[o], bb = a.sb[o], pp = a.sp[o];
+  for (int t = t0; t < t1; t++) {
+    const size_t i = (size_t)t * a.C + c;
+    const float k = a.k[i], v = a.v[i];
+    // kernels/cuda/att.cu:43-60
+    float ww = u + k;
+    float p = (pp > ww) ? pp : ww;
+    float e1 = expf(pp - p), e2 = expf(ww - p);
+    const float wkv = (e1 * aa + e2 * v) / (e1 * bb + e2);
+    a.r[i] = a.r[i] * (h1)wkv;
+    ww = w + pp;
+    p = (ww > k) ? ww : k;
+    e1 = expf(ww - p);
+    e2 = expf(k - p);
+    aa = e1 * aa + e2 * v;
+    bb = e1 * bb + e2;
+    pp = p;
+  }
+  if (ch == a.nchunk - 1) {
+    a.aa_out[c] = aa;
+    a.bb_out[c] = bb;
+    a.pp_out[c] = pp;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// RWKV-5.2 scan, head size 64.  r, k, v [T][C] fp32; state [H][64 key][64 value] fp32.
+// A workgroup of 256 threads serves one (head, chunk): thread t owns value index
+// j = t % 64 and key rows i = (t / 64) * 16 .. +15 of the state (16 registers).
+// Output row t: y_j = sum_i r_i (u_i k_i v_j + s_ij), then groupnorm over the head's 64
+// values, rounding to half and the gate multiply (att_seq.cu:294-316, :406-411).
+// ---------------------------------------------------------------------------
+struct Wkv5Seq {
+  int T, C, H, Lc, nchunk;
+  const float *r, *k, *v, *w, *u, *lx_w, *lx_b;
+  const h1* g;       // [T][C] gate, already through silu
+  const float* s;    // state before the sequence
+  float* loc;        // [nchunk][H][64][64] local end states
+  float* sin;        // [nchunk][H][64][64] state at the start of each chunk
+  float* s_out;
+  h1* gated;         // [T][C]
+};
+
+constexpr int S5 = 64;
+
+__global__ __launch_bounds__(256) void wkv5_local_kernel(Wkv5Seq a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* kk = reinterpret_cast<float*>(smem);  // [Lc][64]
+  float* vv = kk + a.Lc * S5;
+  __shared__ float wsh[S5];
+  const int h = blockIdx.x, ch = blockIdx.y, t = threadIdx.x, j = t & 63, ig = t >> 6;
+  const int t0 = ch * a.Lc, len = min(a.Lc, a.T - t0);
+  for (int e = t; e < len * S5; e += 256) {
+    const size_t src = (size_t)(t0 + e / S5) * a.C + h * S5 + (e % S5);
+    kk[e] = a.k[src];
+    vv[e] = a.v[src];
+  }
+  if (t < S5) wsh[t] = a.w[h * S5 + t];
+  __syncthreads();
+  float s[16];
+#pragma unroll
+  for (int ii = 0; ii < 16; ii++) s[ii] = 0.f;
+  for (int tt = 0; tt < len; tt++) {
+    const float vj = vv[tt * S5 + j];
+#pragma unroll
+    for (int ii = 0; ii < 16; ii++) {
+      const int i = ig * 16 + ii;
+      const float aij = kk[tt * S5 + i] * vj;
+      const float ws = wsh[i] * s[ii];
+      s[ii] = ws + aij;
+    }
+  }
+  float* dst = a.loc + ((size_t)ch * a.H + h) * S5 * S5;
+#pragma unroll
+  for (int ii = 0; ii < 16; ii++) dst[(ig * 16 + ii) * S5 + j] = s[ii];
+}
+
+__global__ __launch_bounds__(256) void wkv5_carry_kernel(Wkv5Seq a) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;  // element of [H][64][64]
+  const size_t per = (size_t)a.H * S5 * S5;
+  if (e >= per) return;
+  const int i = (int)((e / S5) % S5), h = (int)(e / (S5 * S5));
+  const float w = a.w[h * S5 + i];
+  float s = a.s[e];
+  for (int ch = 0; ch < a.nchunk; ch++) {
+    a.sin[(size_t)ch * per + e] = s;
+    const int len = min(a.Lc, a.T - ch * a.Lc);
+    for (int q = 0; q < len; q++) s = w * s;  // decay of the incoming state over the chunk
+    s = s + a.loc[(size_t)ch * per + e];
+  }
+}
+
+__global__ __launch_bounds__(256) void wkv5_apply_kernel(Wkv5Seq a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* rr = reinterpret_cast<float*>(smem);  // [Lc][64]
+  float* kk = rr + a.Lc * S5;
+  float* vv = kk + a.Lc * S5;
+  __shared__ float wsh[S5], ush[S5];
+  __shared__ float part[2][4][S5];
+  const int h = blockIdx.x, ch = blockIdx.y, t = threadIdx.x, j = t & 63, ig = t >> 6;
+  const int t0 = ch * a.Lc, len = min(a.Lc, a.T - t0);
+  for (int e = t; e < len * S5; e += 256) {
+    const size_t src = (size_t)(t0 + e / S5) * a.C + h * S5 + (e % S5);
+    rr[e] = a.r[src];
+    kk[e] = a.k[src];
+    vv[e] = a.v[src];
+  }
+  if (t < S5) {
+    wsh[t] = a.w[h * S5 + t];
+    ush[t] = a.u[h * S5 + t];
+  }
+  const float* src = a.sin + ((size_t)ch * a.H + h) * S5 * S5;
+  float s[16];
+#pragma unroll
+  for (int ii = 0; ii < 16; ii++) s[ii] = src[(ig * 16 + ii) * S5 + j];
+  float gw = 0.f, gb = 0.f;
+  if (t < S5) {
+    gw = a.lx_w[h * S5 + t];
+    gb = a.lx_b[h * S5 + t];
+  }
+  __syncthreads();
+  for (int tt = 0; tt < len; tt++) {
+    const float vj = vv[tt * S5 + j];
+    float acc = 0.f;
+#pragma unroll
+    for (int ii = 0; ii < 16; ii++) {
+      const int i = ig * 16 + ii;
+      const float aij = kk[tt * S5 + i] * vj;
+      const float ua = ush[i] * aij;
+      const float tmp = ua + s[ii];
+      const float ws = wsh[i] * s[ii];
+      s[ii] = ws + aij;
+      acc += rr[tt * S5 + i] * tmp;
+    }
+    part[tt & 1][ig][j] = acc;
+    __syncthreads();  // the other half of `part` is free again: its readers passed this barrier a step ago
+    if (t < S5) {
+      const float o = ((part[tt & 1][0][t] + part[tt & 1][1][t]) + part[tt & 1][2][t]) + part[tt & 1][3][t];
+      const float mean = wave_sum(o) / (float)S5;
+      const float d = o - mean;
+      float var = wave_sum(d * d) / (float)S5;
+      var = var > 0.f ? var : 0.f;
+      const float inv = 1.0f / sqrtf(var + 1e-5f);
+      const float y = d * inv * gw + gb;
+      const size_t oi = (size_t)(t0 + tt) * a.C + h * S5 + t;
+      a.gated[oi] = (h1)y * a.g[oi];
+    }
+  }
+  if (ch == a.nchunk - 1) {
+    float* dst = a.s_out + (size_t)h * S5 * S5;
+#pragma unroll
+    for (int ii = 0; ii < 16; ii++) dst[(ig * 16 + ii) * S5 + j] = s[ii];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+#define FR_TRY(expr)        \
+  do {                      \
+    int _e = (expr);        \
+    if (_e != 0) return _e; \
+  } while (0)
+
+static size_t al256(size_t n) { return (n + 255) / 256 * 256; }
+
+static int check_w(const frhip_weight* w, int K, int N, const char* what) {
+  if (!w || !w->data) return set_error(FRHIP_EINVAL, what);
+  if (w->dtype != FRHIP_F16 && w->dtype != FRHIP_U8) return set_error(FRHIP_EINVAL, what);
+  if (w->K != K || w->N != N) return set_error(FRHIP_ESHAPE, what);
+  if (w->dtype == FRHIP_U8 && (!w->mx || !w->rx || !w->my || !w->ry)) return set_error(FRHIP_EINVAL, what);
+  return 0;
+}
+
+static int launch_ln_mix(int T, int C, const void* x, const void* state, const void* ln_w, const void* ln_b,
+                         const void* const* mix, h1* const* out, int nmix, void* xx_last, hipStream_t st) {
+  LnMixSeq a;
+  a.T = T; a.C = C; a.nmix = nmix;
+  a.x = (const h1*)x; a.state = (const h1*)state; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+  for (int i = 0; i < nmix; i++) {
+    a.mix[i] = (const h1*)mix[i];
+    a.out[i] = out[i];
+  }
+  a.xx_last = (h1*)xx_last;
+  hipLaunchKernelGGL(ln_mix_seq_kernel, dim3(T), dim3(256), 4 * (size_t)C, st, a);
+  return check_launch("ln_mix_seq");
+}
+
+// chunk length for a scan of T steps when one chunk occupies `units` workgroup-sized units:
+// enough chunks to fill the device (~4 units per CU), chunks of at least 8 steps
+static int pick_chunk(int T, int units) {
+  int want = (4 * compute_units() + units - 1) / units;
+  if (want < 1) want = 1;
+  int Lc = (T + want - 1) / want;
+  if (Lc < 8) Lc = 8;
+  if (Lc > 64) Lc = 64;
+  return Lc;
+}
+
+}  // namespace frhip
+
+using namespace frhip;
+
+extern "C" size_t frhip_seq_workspace_bytes(int T, int C, int F) {
+  if (T <= 0 || C <= 0 || F <= 0) return 0;
+  const size_t tc = (size_t)T * C;
+  // activations: 4 mixed inputs + g + gated (half), k v r y (fp32), vx [T][F] (half)
+  size_t n = 6 * al256(2 * tc) + 4 * al256(4 * tc) + al256(2 * (size_t)T * F);
+  // scan scratch: RWKV-4 6 x [nchunk][C] fp32 with nchunk <= T/8+1; RWKV-5 2 x [nchunk][C*64] fp32
+  const size_t nchunk = (size_t)T / 8 + 1;
+  n += 6 * al256(4 * nchunk * C) + 2 * al256(4 * nchunk * (size_t)C * 64);
+  return n;
+}
+
+namespace {
+struct SeqWs {
+  h1 *m0, *m1, *m2, *m3, *g, *gated, *vx;
+  float *f0, *f1, *f2, *f3;
+  float* scan;
+};
+SeqWs carve_seq(void* ws, int T, int C, int F) {
+  const size_t tc = (size_t)T * C;
+  unsigned char* p = static_cast<unsigned char*>(ws);
+  SeqWs w;
+  h1** hs[6] = {&w.m0, &w.m1, &w.m2, &w.m3, &w.g, &w.gated};
+  for (auto h : hs) {
+    *h = reinterpret_cast<h1*>(p);
+    p += al256(2 * tc);
+  }
+  float** fs[4] = {&w.f0, &w.f1, &w.f2, &w.f3};
+  for (auto f : fs) {
+    *f = reinterpret_cast<float*>(p);
+    p += al256(4 * tc);
+  }
+  w.vx = reinterpret_cast<h1*>(p);
+  p += al256(2 * (size_t)T * F);
+  w.scan = reinterpret_cast<float*>(p);
+  return w;
+}
+}  // namespace
+
+// ffn_seq (kernels/cuda/ffn_seq.cu:65-109).  x [T][C]; sx [C] shift state; xx_out [C] = LN(x)[T-1].
+extern "C" int frhip_ffn_seq(int T, int C, int F, const void* x, const void* sx, const void* ln_w, const void* ln_b,
+                             const void* k_mix, const void* r_mix, const frhip_weight* kw, const frhip_weight* vw,
+                             const frhip_weight* rw, void* x_out, void* xx_out, int post_div2, void* workspace,
+                             frhip_stream s) {
+  if (T <= 0) return set_error(FRHIP_ESHAPE, "ffn_seq: T must be positive");
+  if (!x || !sx || !ln_w || !ln_b || !k_mix || !r_mix || !x_out || !xx_out || !workspace)
+    return set_error(FRHIP_EINVAL, "ffn_seq: null pointer");
+  if (C <= 0 || C % 64 != 0 || F <= 0 || F % 64 != 0) return set_error(FRHIP_ESHAPE, "ffn_seq: C and F must be multiples of 64");
+  FR_TRY(check_w(kw, C, F, "ffn_seq: bad key weight"));
+  FR_TRY(check_w(vw, F, C, "ffn_seq: bad value weight"));
+  FR_TRY(check_w(rw, C, C, "ffn_seq: bad receptance weight"));
+  hipStream_t st = static_cast<hipStream_t>(s);
+  SeqWs w = carve_seq(workspace, T, C, F);
+  const void* mixes[2] = {k_mix, r_mix};
+  h1* outs[2] = {w.m0, w.m1};
+  FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, 2, xx_out, st));
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = T; a.K = C;
+  gemm_add_seg(a, w.m1, rw, w.m2, G_SIGMOID);  // r
+  gemm_add_seg(a, w.m0, kw, w.vx, G_RELU2);    // vx
+  if (kw->dtype != rw->dtype) return set_error(FRHIP_EINVAL, "ffn_seq: key/receptance dtypes differ");
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "ffn_seq r,k"));
+  GemmArgs b;
+  memset(&b, 0, sizeof(b));
+  b.M = T; b.K = F;
+  b.res_x = (const h1*)x; b.res_r = w.m2; b.div2 = post_div2 ? 1 : 0;
+  gemm_add_seg(b, w.vx, vw, x_out, G_FFN_OUT);
+  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v");
+}
+
+// RWKV-4 sequence attention.  The reference has no such operator
+// (kernels/default/model_forward_seq.cpp:111-112); the result is defined by T one-token steps
+// of kernels/cuda/att.cu:182-217 (model_forward_seq.cpp:34-46).
+extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, const float* aa, const float* bb,
+                                const float* pp, const void* ln_w, const void* ln_b, const void* k_mix,
+                                const void* v_mix, const void* r_mix, const float* t_decay, const float* t_first,
+                                const frhip_weight* kw, const frhip_weight* vw, const frhip_weight* rw,
+                                const frhip_weight* ow, void* x_out, void* xx_out, float* aa_out, float* bb_out,
+                                float* pp_out, void* workspace, frhip_stream s) {
+  if (T <= 0) return set_error(FRHIP_ESHAPE, "att_seq_v4: T must be positive");
+  if (!x || !sx || !aa || !bb || !pp || !ln_w || !ln_b || !k_mix || !v_mix || !r_mix || !t_decay || !t_first ||
+      !x_out || !xx_out || !aa_out || !bb_out || !pp_out || !workspace)
+    return set_error(FRHIP_EINVAL, "att_seq_v4: null pointer");
+  if (C <= 0 || C % 64 != 0) return set_error(FRHIP_ESHAPE, "att_seq_v4: C must be a multiple of 64");
+  FR_TRY(check_w(kw, C, C, "att_seq_v4: bad key weight"));
+  FR_TRY(check_w(vw, C, C, "att_seq_v4: bad value weight"));
+  FR_TRY(check_w(rw, C, C, "att_seq_v4: bad receptance weight"));
+  FR_TRY(check_w(ow, C, C, "att_seq_v4: bad output weight"));
+  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype) return set_error(FRHIP_EINVAL, "att_seq_v4: k/v/r dtypes differ");
+  hipStream_t st = static_cast<hipStream_t>(s);
+  SeqWs w = carve_seq(workspace, T, C, 64);
+  const void* mixes[3] = {k_mix, v_mix, r_mix};
+  h1* outs[3] = {w.m0, w.m1, w.m2};
+  FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, 3, xx_out, st));
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = T; a.K = C;
+  gemm_add_seg(a, w.m0, kw, w.f0, G_STORE_F32);  // k
+  gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
+  gemm_add_seg(a, w.m2, rw, w.m3, G_SIGMOID);    // r
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v4 k,v,r"));
+
+  Wkv4Seq q;
+  q.T = T; q.C = C;
+  q.Lc = pick_chunk(T, (C + 255) / 256);
+  q.nchunk = (T + q.Lc - 1) / q.Lc;
+  q.k = w.f0; q.v = w.f1; q.u = t_first; q.w = t_decay; q.r = w.m3;
+  q.aa = aa; q.bb = bb; q.pp = pp;
+  const size_t n = al256(4 * (size_t)q.nchunk * C) / 4;
+  q.la = w.scan; q.lb = q.la + n; q.lp = q.lb + n; q.sa = q.lp + n; q.sb = q.sa + n; q.sp = q.sb + n;
+  q.aa_out = aa_out; q.bb_out = bb_out; q.pp_out = pp_out;
+  dim3 grid((C + 255) / 256, q.nchunk);
+  hipLaunchKernelGGL(wkv4_local_kernel, grid, dim3(256), 0, st, q);
+  hipLaunchKernelGGL(wkv4_carry_kernel, dim3((C + 255) / 256), dim3(256), 0, st, q);
+  hipLaunchKernelGGL(wkv4_apply_kernel, grid, dim3(256), 0, st, q);
+  FR_TRY(check_launch("wkv4_seq"));
+
+  GemmArgs b;
+  memset(&b, 0, sizeof(b));
+  b.M = T; b.K = C;
+  b.res_x = (const h1*)x;
+  gemm_add_seg(b, w.m3, ow, x_out, G_RESIDUAL);
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v4 out");
+}
+
+// att_seq_v5_2 (kernels/cuda/att_seq.cu:368-423,464-493).
+extern "C" int frhip_att_seq_v5_2(int T, int C, int H, const void* x, const void* sx, const float* s_in,
+                                  const void* ln_w, const void* ln_b, const float* lx_w, const float* lx_b,
+                                  const void* k_mix, const void* v_mix, const void* r_mix, const void* g_mix,
+                                  const float* t_decay, const float* t_first, const frhip_weight* kw,
+                                  const frhip_weight* vw, const frhip_weight* rw, const frhip_weight* gw,
+                                  const frhip_weight* ow, void* x_out, void* xx_out, float* s_out, void* workspace,
+                                  frhip_stream s) {
+  if (T <= 0) return set_error(FRHIP_ESHAPE, "att_seq_v5_2: T must be positive");
+  if (!x || !sx || !s_in || !ln_w || !ln_b || !lx_w || !lx_b || !k_mix || !v_mix || !r_mix || !g_mix || !t_decay ||
+      !t_first || !x_out || !xx_out || !s_out || !workspace)
+    return set_error(FRHIP_EINVAL, "att_seq_v5_2: null pointer");
+  if (H <= 0 || C % H != 0 || C / H != 64) return set_error(FRHIP_ESHAPE, "att_seq_v5_2: head size must be 64");
+  FR_TRY(check_w(kw, C, C, "att_seq_v5_2: bad key weight"));
+  FR_TRY(check_w(vw, C, C, "att_seq_v5_2: bad value weight"));
+  FR_TRY(check_w(rw, C, C, "att_seq_v5_2: bad receptance weight"));
+  FR_TRY(check_w(gw, C, C, "att_seq_v5_2: bad gate weight"));
+  FR_TRY(check_w(ow, C, C, "att_seq_v5_2: bad output weight"));
+  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype || kw->dtype != gw->dtype)
+    return set_error(FRHIP_EINVAL, "att_seq_v5_2: k/v/r/g dtypes differ");
+  hipStream_t st = static_cast<hipStream_t>(s);
+  SeqWs w = carve_seq(workspace, T, C, 64);
+  const void* mixes[4] = {k_mix, v_mix, r_mix, g_mix};
+  h1* outs[4] = {w.m0, w.m1, w.m2, w.m3};
+  FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, 4, xx_out, st));
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = T; a.K = C;
+  gemm_add_seg(a, w.m0, kw, w.f0, G_STORE_F32);  // k
+  gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
+  gemm_add_seg(a, w.m2, rw, w.f2, G_STORE_F32);  // r
+  gemm_add_seg(a, w.m3, gw, w.g, G_SILU);        // g
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5_2 k,v,r,g"));
+
+  Wkv5Seq q;
+  q.T = T; q.C = C; q.H = H;
+  q.Lc = pick_chunk(T, H);
+  q.nchunk = (T + q.Lc - 1) / q.Lc;
+  q.r = w.f2; q.k = w.f0; q.v = w.f1; q.w = t_decay; q.u = t_first; q.lx_w = lx_w; q.lx_b = lx_b;
+  q.g = w.g; q.s = s_in; q.s_out = s_out; q.gated = w.gated;
+  const size_t per = al256(4 * (size_t)q.nchunk * C * 64) / 4;
+  q.loc = w.scan;
+  q.sin = q.loc + per;
+  dim3 grid(H, q.nchunk);
+  hipLaunchKernelGGL(wkv5_local_kernel, grid, dim3(256), 2 * sizeof(float) * q.Lc * S5, st, q);
+  hipLaunchKernelGGL(wkv5_carry_kernel, dim3(((size_t)H * S5 * S5 + 255) / 256), dim3(256), 0, st, q);
+  hipLaunchKernelGGL(wkv5_apply_kernel, grid, dim3(256), 3 * sizeof(float) * q.Lc * S5, st, q);
+  FR_TRY(check_launch("wkv5_seq"));
+
+  GemmArgs b;
+  memset(&b, 0, sizeof(b));
+  b.M = T; b.K = C;
+  b.res_x = (const h1*)x;
+  gemm_add_seg(b, w.gated, ow, x_out, G_RESIDUAL);
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5_2 out");
+}

@@ -14,6 +14,7 @@
 // FR_HIP_GENERIC=1 selects the operator-by-operator loop instead; FR_HIP_NO_GRAPH=1 keeps
 // the fused path but launches eagerly.
 #include <cstdlib>
+#include <cstring>
 
 #include "kernels/hip/context.h"
 #include "kernels/hip/hip_model.h"
@@ -218,8 +219,58 @@ Tensor ModelForward(Model *model, Device device, int id) {
   return Tensor::FromPtr(p.logits_host[cur], {p.n_logits}, DType::kFloat32, Device::kCPU);
 }
 
+// Seq mode (reference: kernels/default/model_forward_seq.cpp:48-184): embedding rows are
+// gathered on the device, every layer runs its seq operator over all T rows (MFMA products,
+// chunked WKV scans), and only the last row goes through ln_out and the head.  RWKV-4, which
+// upstream cannot run in seq mode (:111-112), goes through the `att_seq` operator.
+// FR_HIP_SEQ_FALLBACK=1 selects the loop of one-token steps (:34-46) instead.
 Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids, bool full_output) {
-  return def::ModelForwardSeqFallback(model, device, ids, full_output);
+  const std::string &ver = model->version();
+  if (std::getenv("FR_HIP_SEQ_FALLBACK") || !(ver == "4" || ver == "5.2"))
+    return def::ModelForwardSeqFallback(model, device, ids, full_output);
+  RV_CHECK(!full_output) << "full_output is not supported on hip yet";
+  RV_CHECK(!ids.empty());
+  auto ex = extra_of(model);
+  const int T = static_cast<int>(ids.size()), C = model->n_embd();
+  const int V = static_cast<int>(ex->emb_table.size(0));
+  for (int id : ids) RV_CHECK(id >= 0 && id < V) << "token id " << id << " out of range";
+  frhip_stream s = stream();
+  // ids -> device -> gather (reference: vgather, T separate device copies)
+  Tensor ids_cpu = Tensor::Empty({T}, DType::kInt32, Device::kCPU);
+  std::memcpy(ids_cpu.data_ptr(), ids.data(), sizeof(int32_t) * ids.size());
+  Tensor ids_dev = Copy(ids_cpu, Device::kHIP, true);
+  Tensor x = Tensor::Empty({T, C}, DType::kFloat16, Device::kHIP);
+  FRHIP_CHECK(frhip_gather_rows(ex->emb_table.data_ptr(), ids_dev.data_ptr<int32_t>(), x.data_ptr(), T, 2 * C, s));
+
+  auto &states = model->states();
+  const auto &p = model->_params;
+  size_t pi = 0;
+  for (size_t i = 0; i < states.size(); i++) {
+    auto &st = states[i];
+    if (ver == "4") {
+      std::tie(x, st[0], st[1], st[2], st[3]) =
+          att_seq(x, st[0], st[1], st[2], st[3], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5],
+                  p[pi + 6], p[pi + 7], p[pi + 8], p[pi + 9], p[pi + 10]);
+      pi += 11;
+    } else {
+      std::tie(x, st[0], st[1]) =
+          att_seq_v5_2(x, st[0], st[1], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5], p[pi + 6],
+                       p[pi + 7], p[pi + 8], p[pi + 9], p[pi + 10], p[pi + 11], p[pi + 12], p[pi + 13], p[pi + 14],
+                       model->n_att());
+      pi += 15;
+    }
+    const int off = ver[0] == '5' ? 2 : 4;
+    std::tie(x, st[off]) = ffn_seq(x, st[off], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5], p[pi + 6]);
+    pi += 7;
+    if ((i + 1) % 6 == 0) scalar_div_(x, 2);
+  }
+  // last row -> ln_out -> head -> fp32 (model_forward_seq.cpp:170-178)
+  const frhip_weight *hw = find_weight(p[pi + 2]);
+  RV_CHECK(hw != nullptr);
+  Tensor logits = Tensor::Empty({static_cast<LengthType>(hw->N)}, DType::kFloat32, Device::kHIP);
+  const char *last = static_cast<const char *>(x.data_ptr()) + static_cast<size_t>(T - 1) * C * 2;
+  FRHIP_CHECK(frhip_head(C, last, p[pi].data_ptr(), p[pi + 1].data_ptr(), hw, logits.data_ptr<float>(), s));
+  return logits;
 }
 
 KernelRegister model_forward_reg("model_forward", Device::kHIP, ModelForward);

@@ -186,6 +186,80 @@ att_one_v5_1(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &l
   return {x_out, xx, s_out};
 }
 
+static Tensor seq_workspace(int T, int C, int F) {
+  return Tensor::Empty({static_cast<LengthType>(frhip_seq_workspace_bytes(T, C, F))}, DType::kInt8, Device::kHIP);
+}
+
+// ffn_seq (reference: kernels/cuda/ffn_seq.cu:89-109).  x [T, C]; returns (x_out [T, C], LN(x)[T-1]).
+std::tuple<Tensor, Tensor> ffn_seq(const Tensor &x, const Tensor &sx, const Tensor &ln_w, const Tensor &ln_b,
+                                   const Tensor &k_mix, const Tensor &r_mix, const Tensor &kw, const Tensor &vw,
+                                   const Tensor &rw) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 2);
+  const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1)), F = static_cast<int>(kw.size(1));
+  frhip_weight d[3];
+  Tensor tmp[3];
+  const frhip_weight *w[3] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
+  Tensor ws = seq_workspace(T, C, F);
+  FRHIP_CHECK(frhip_ffn_seq(T, C, F, x.data_ptr(), sx.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), k_mix.data_ptr(),
+                            r_mix.data_ptr(), w[0], w[1], w[2], x_out.data_ptr(), xx.data_ptr(), 0, ws.data_ptr(),
+                            stream()));
+  return {x_out, xx};
+}
+
+// att_seq, RWKV-4 (no counterpart upstream: kernels/default/model_forward_seq.cpp:111-112 throws).
+std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor>
+att_seq(const Tensor &x, const Tensor &sx, const Tensor &aa, const Tensor &bb, const Tensor &pp, const Tensor &ln_w,
+        const Tensor &ln_b, const Tensor &k_mix, const Tensor &v_mix, const Tensor &r_mix, const Tensor &t_decay,
+        const Tensor &t_first, const Tensor &kw, const Tensor &vw, const Tensor &rw, const Tensor &ow) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 2);
+  const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1));
+  frhip_weight d[4];
+  Tensor tmp[4];
+  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
+                              weight_of(ow, d[3], tmp[3])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
+  Tensor t1 = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor t2 = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor p = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor ws = seq_workspace(T, C, 64);
+  FRHIP_CHECK(frhip_att_seq_v4(T, C, x.data_ptr(), sx.data_ptr(), aa.data_ptr<float>(), bb.data_ptr<float>(),
+                               pp.data_ptr<float>(), ln_w.data_ptr(), ln_b.data_ptr(), k_mix.data_ptr(),
+                               v_mix.data_ptr(), r_mix.data_ptr(), t_decay.data_ptr<float>(),
+                               t_first.data_ptr<float>(), w[0], w[1], w[2], w[3], x_out.data_ptr(), xx.data_ptr(),
+                               t1.data_ptr<float>(), t2.data_ptr<float>(), p.data_ptr<float>(), ws.data_ptr(),
+                               stream()));
+  return {x_out, xx, t1, t2, p};
+}
+
+// att_seq_v5_2 (reference: kernels/cuda/att_seq.cu:464-493).
+std::tuple<Tensor, Tensor, Tensor>
+att_seq_v5_2(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &ln_w, const Tensor &ln_b,
+             const Tensor &lx_w, const Tensor &lx_b, const Tensor &k_mix, const Tensor &v_mix, const Tensor &r_mix,
+             const Tensor &g_mix, const Tensor &t_decay, const Tensor &t_first, const Tensor &kw, const Tensor &vw,
+             const Tensor &rw, const Tensor &gw, const Tensor &ow, int n_att) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 2);
+  const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1));
+  RV_CHECK(n_att == C) << "att_seq_v5_2 on hip: n_att must equal n_embd";
+  const int H = static_cast<int>(t_decay.size(0));
+  frhip_weight d[5];
+  Tensor tmp[5];
+  const frhip_weight *w[5] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
+                              weight_of(gw, d[3], tmp[3]), weight_of(ow, d[4], tmp[4])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
+  Tensor s_out = Tensor::Empty(s.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor ws = seq_workspace(T, C, 64);
+  FRHIP_CHECK(frhip_att_seq_v5_2(T, C, H, x.data_ptr(), sx.data_ptr(), s.data_ptr<float>(), ln_w.data_ptr(),
+                                 ln_b.data_ptr(), lx_w.data_ptr<float>(), lx_b.data_ptr<float>(), k_mix.data_ptr(),
+                                 v_mix.data_ptr(), r_mix.data_ptr(), g_mix.data_ptr(), t_decay.data_ptr<float>(),
+                                 t_first.data_ptr<float>(), w[0], w[1], w[2], w[3], w[4], x_out.data_ptr(),
+                                 xx.data_ptr(), s_out.data_ptr<float>(), ws.data_ptr(), stream()));
+  return {x_out, xx, s_out};
+}
+
 KernelRegister fill_reg("fill_", Device::kHIP, fill_);
 KernelRegister cast_reg("cast_dtype", Device::kHIP, cast_dtype);
 KernelRegister scalar_div_reg("scalar_div_", Device::kHIP, scalar_div_);
@@ -195,6 +269,9 @@ KernelRegister matmul_reg("matmul", Device::kHIP, matmul);
 KernelRegister vgather_reg("vgather", Device::kHIP, vgather);
 KernelRegister att_reg("att", Device::kHIP, att);
 KernelRegister ffn_reg("ffn", Device::kHIP, ffn);
+KernelRegister ffn_seq_reg("ffn_seq", Device::kHIP, ffn_seq);
+KernelRegister att_seq_reg("att_seq", Device::kHIP, att_seq);
+KernelRegister att_seq_v5_2_reg("att_seq_v5_2", Device::kHIP, att_seq_v5_2);
 KernelRegister att_one_v5_1_reg("att_one_v5_1", Device::kHIP, att_one_v5_1);
 
 }  // namespace hip

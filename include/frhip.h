@@ -159,6 +159,45 @@ int frhip_att_one_v5_1(int C, int H, const void *x, const void *sx, const float 
                        const frhip_weight *gw, const frhip_weight *ow,
                        void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
 
+/* ---- seq-mode (prompt) operators ---------------------------------------------- */
+/* matmul, matrix x matrix: kernels/cuda/matmul.cpp:110-121.  x [T][K] binary16, y [T][N] in
+ * out_dtype (F16 or F32); fp32 accumulation on the MFMA units.  K must be a multiple of 64. */
+int frhip_gemm(const void *x, const frhip_weight *w, void *y, int T, int out_dtype, frhip_stream s);
+
+/* Scratch for the seq-mode operators below: frhip_seq_workspace_bytes(T, C, F) bytes,
+ * 256-byte aligned, owned by the caller. */
+size_t frhip_seq_workspace_bytes(int T, int C, int F);
+
+/* ffn_seq: kernels/cuda/ffn_seq.cu:65-109.  x, x_out [T][C]; sx [C]; xx_out [C] receives
+ * LN(x)[T-1], the new shift state.  post_div2 as in frhip_ffn_one.  x_out may alias x. */
+int frhip_ffn_seq(int T, int C, int F, const void *x, const void *sx, const void *ln_w, const void *ln_b,
+                  const void *k_mix, const void *r_mix,
+                  const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                  void *x_out, void *xx_out, int post_div2, void *workspace, frhip_stream s);
+
+/* att_seq for RWKV-4.  The reference has no seq-mode att for version 4
+ * (kernels/default/model_forward_seq.cpp:111-112 throws); its fallback
+ * (model_forward_seq.cpp:34-46) defines the result as T one-token att steps
+ * (kernels/cuda/att.cu:182-217), which is what this computes, with the products batched
+ * over T and the WKV recurrence run as a chunked scan.  State arguments as frhip_att_one_v4. */
+int frhip_att_seq_v4(int T, int C, const void *x, const void *sx, const float *aa, const float *bb, const float *pp,
+                     const void *ln_w, const void *ln_b, const void *k_mix, const void *v_mix, const void *r_mix,
+                     const float *t_decay, const float *t_first,
+                     const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw, const frhip_weight *ow,
+                     void *x_out, void *xx_out, float *aa_out, float *bb_out, float *pp_out,
+                     void *workspace, frhip_stream s);
+
+/* att_seq_v5_2: kernels/cuda/att_seq.cu:368-423,464-493.  State [H][S][S] indexed
+ * [head][key][value] as in frhip_att_one_v5_1 (the reference transposes it around its scan
+ * kernel, att_seq.cu:397,404; here the scan indexes it directly).  s_out may alias s. */
+int frhip_att_seq_v5_2(int T, int C, int H, const void *x, const void *sx, const float *s,
+                       const void *ln_w, const void *ln_b, const float *lx_w, const float *lx_b,
+                       const void *k_mix, const void *v_mix, const void *r_mix, const void *g_mix,
+                       const float *t_decay, const float *t_first,
+                       const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                       const frhip_weight *gw, const frhip_weight *ow,
+                       void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
+
 /* greedy sampler step (Sampler::Sample with top_k = 1, chat.cpp:76-77): index of the
  * largest logit, first one on ties, written to *out_id on the device. */
 int frhip_argmax_f32(const float *logits, int n, int32_t *out_id, frhip_stream s);

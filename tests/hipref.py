@@ -24,15 +24,17 @@ def ulp_diff_f16(a, b):
     return np.abs(key(a) - key(b))
 
 
-def assert_close_f16(got, ref, max_ulp=2, max_frac=0.03, what=""):
+def assert_close_f16(got, ref, max_ulp=2, max_frac=0.03, what="", floor_rms=0.25):
     """|got-ref| <= max_ulp binary16 spacings, the spacing taken at max(|ref|, rms(ref)/4):
     an output formed by cancellation (x + out close to 0) inherits the absolute rounding
-    error of its operands, which is not small in units of its own tiny spacing."""
+    error of its operands, which is not small in units of its own tiny spacing.  floor_rms
+    raises that floor for outputs whose operands are larger than the output itself (the
+    ffn product can be several times the residual it is added to)."""
     got, ref = np.asarray(got, np.float16), np.asarray(ref, np.float16)
     assert got.shape == ref.shape, (got.shape, ref.shape)
     g32, r32 = got.astype(np.float32), ref.astype(np.float32)
     assert np.isfinite(g32).all(), what + ": non-finite output"
-    floor = 0.25 * float(np.sqrt(np.mean(r32.astype(np.float64) ** 2))) + 1e-6
+    floor = floor_rms * float(np.sqrt(np.mean(r32.astype(np.float64) ** 2))) + 1e-6
     mag = np.maximum(np.abs(r32), floor)
     spacing = np.exp2(np.floor(np.log2(mag)) - 10)
     err = np.abs(g32 - r32)

@@ -91,16 +91,26 @@ def test_reset_and_state_file_round_trip(model_files, tmp_path):
     m.close()
 
 
-def test_seq_mode_equals_one_token_steps(model_files):
-    """kernels/default/model_forward_seq.cpp:34-46: Run(ids) == Run(id) for each id."""
-    path, _, _ = model_files
-    ids = [5, 17, 299, 0, 42, 7, 7, 123]
-    m = fr.Model(path, "hip fp16")
+@pytest.mark.parametrize("strategy", ["hip fp16", "hip int8"])
+def test_seq_mode_equals_one_token_steps_and_oracle(model_files, strategy):
+    """kernels/default/model_forward_seq.cpp:34-46: Run(ids) == Run(id) for each id -- for
+    logits AND for the state left behind (checked by continuing to decode from it)."""
+    path, params, emb = model_files
+    ids = [int(t) for t in np.random.default_rng(43).integers(0, V_, 200)]
+    m = fr.Model(path, strategy)
     seq = m.run(ids)
+    after_seq = [m.run(t) for t in (9, 8, 7)]
     m.reset()
     for i in ids:
         one = m.run(i)
+    after_one = [m.run(t) for t in (9, 8, 7)]
     assert np.abs(seq - one).max() <= 2e-2
+    assert int(np.argmax(seq)) == int(np.argmax(one))
+    for a, b in zip(after_seq, after_one):
+        assert np.abs(a - b).max() <= 2e-2
+    om = _oracle(params, emb, strategy.endswith("int8"))
+    ref = om.run(ids)
+    assert np.abs(seq - ref).max() <= 2e-2 and int(np.argmax(seq)) == int(np.argmax(ref))
     m.close()
 
 
@@ -149,4 +159,15 @@ def test_rwkv5_2_model_matches_oracle(tmp_path):
         s_ref = om.state[5 * 3 + 1]
         s_got = m.state(5, 1, np.float32)
         assert np.abs(s_got - s_ref).max() <= 5e-3 * np.abs(s_ref).max()
+        # seq-mode prefill of a prompt, then decode: same logits as the oracle's seq mode
+        m.reset()
+        om.reset()
+        prompt = [int(t) for t in np.random.default_rng(44).integers(0, V5, 96)]
+        ls, lo = m.run(prompt), om.run(prompt)
+        assert np.abs(ls - lo).max() <= 2e-2 and int(np.argmax(ls)) == int(np.argmax(lo))
+        tok = int(np.argmax(lo))
+        for step in range(8):
+            ls, lo = m.run(tok), om.run(tok)
+            assert np.abs(ls - lo).max() <= 2e-2
+            tok = int(np.argmax(lo))
         m.close()

@@ -1,0 +1,158 @@
+"""GPU parity tests of the seq-mode (prompt) operators against the oracle."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import pyoracle as po
+from hipref import DevBuf, L, assert_close_f16, dev, fr, make_weight
+
+_alive = []
+
+
+def keep(a):
+    b = dev(a)
+    _alive.append(b)
+    if len(_alive) > 96:
+        fr.check(L().frhip_device_sync())
+        del _alive[:48]
+    return b
+
+
+rng = np.random.default_rng(777)
+
+
+def h(x):
+    return np.asarray(x, np.float32).astype(np.float16)
+
+
+@pytest.mark.parametrize("T,K,N", [(1024, 2048, 2048), (512, 2560, 8960), (100, 8192, 2048), (1, 64, 128), (130, 128, 200), (7, 1792, 512)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_gemm_against_oracle(T, K, N, quant):
+    x = h(rng.standard_normal((T, K)))
+    w = h(rng.standard_normal((K, N)) * 0.02)
+    pw, wref = make_weight(w, quant)
+    ref = po.gemm_f16(x, wref, "f32")
+    y32, y16 = DevBuf.empty((T, N), np.float32), DevBuf.empty((T, N), np.float16)
+    fr.check(L().frhip_gemm(keep(x).ptr, pw.ref, y32.ptr, T, fr.F32, None))
+    fr.check(L().frhip_gemm(keep(x).ptr, pw.ref, y16.ptr, T, fr.F16, None))
+    got = y32.numpy()
+    tol = 3e-6 * np.sqrt(K) * np.abs(ref).max() + 1e-5
+    assert np.abs(got - ref).max() <= tol, np.abs(got - ref).max()
+    assert_close_f16(y16.numpy(), ref.astype(np.float16), max_ulp=1, what="gemm f16 out")
+    # an asymmetric probe: row t = e_k picks out row k of the weight exactly (catches a swapped
+    # operand or a wrong fragment layout that a random comparison could only show as noise)
+    if T >= 4:
+        e = np.zeros((T, K), np.float16)
+        ks = [0, 1, K // 2 + 3, K - 1]
+        for t, k in enumerate(ks):
+            e[t, k] = 1
+        fr.check(L().frhip_gemm(keep(e).ptr, pw.ref, y32.ptr, T, fr.F32, None))
+        out = y32.numpy()
+        for t, k in enumerate(ks):
+            assert np.array_equal(out[t], wref[k].astype(np.float32)), (t, k)
+        assert not out[len(ks):].any()
+
+
+def test_gemm_rejects_bad_shapes():
+    w = fr.PackedWeight(w_kn=h(rng.standard_normal((96, 64))))
+    y = DevBuf.empty((4, 64), np.float32)
+    assert L().frhip_gemm(keep(h(np.zeros((4, 96)))).ptr, w.ref, y.ptr, 4, fr.F32, None) == -2  # K % 64
+    assert L().frhip_gemm(None, w.ref, y.ptr, 4, fr.F32, None) == -1
+
+
+def _common(C_):
+    return (h(1 + 0.1 * rng.standard_normal(C_)), h(0.1 * rng.standard_normal(C_)))
+
+
+@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1, 512, 1024), (33, 768, 3072)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_ffn_seq(T, C_, F_, quant):
+    if quant and C_ == 2048:
+        pytest.skip("covered by the fp16 case at this size; uint8 covered at the smaller sizes")
+    x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
+    ln_w, ln_b = _common(C_)
+    mk, mr = h(rng.uniform(0, 1, C_)), h(rng.uniform(0, 1, C_))
+    kw, kref = make_weight(h(rng.standard_normal((C_, F_)) * 0.02), quant)
+    vw, vref = make_weight(h(rng.standard_normal((F_, C_)) * 0.02), quant)
+    rw, rref = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+    ref_x, ref_xx = po.ffn_f16(x, sx, ln_w, ln_b, mk, mr, kref, vref, rref)
+    x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
+    ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, F_))
+    fr.check(L().frhip_ffn_seq(T, C_, F_, keep(x).ptr, keep(sx).ptr, keep(ln_w).ptr, keep(ln_b).ptr, keep(mk).ptr,
+                               keep(mr).ptr, kw.ref, vw.ref, rw.ref, x_out.ptr, xx_out.ptr, 0, ws.ptr, None))
+    assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx_last")
+    assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out", floor_rms=1.0)
+
+
+def _state_v4(C_, fresh):
+    if fresh:
+        return np.zeros(C_, np.float32), np.zeros(C_, np.float32), np.full(C_, -1e30, np.float32)
+    return (rng.standard_normal(C_).astype(np.float32), rng.uniform(0.5, 3, C_).astype(np.float32),
+            rng.standard_normal(C_).astype(np.float32))
+
+
+@pytest.mark.parametrize("T,C_", [(64, 512), (1024, 2048), (1, 512), (37, 768)])
+@pytest.mark.parametrize("quant", [False, True])
+@pytest.mark.parametrize("fresh", [True, False])
+def test_att_seq_v4(T, C_, quant, fresh):
+    if C_ == 2048 and (quant or not fresh):
+        pytest.skip("full-size case runs once")
+    x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
+    aa, bb, pp = _state_v4(C_, fresh)
+    ln_w, ln_b = _common(C_)
+    mixes = [h(rng.uniform(0, 1, C_)) for _ in range(3)]
+    td = (-np.exp(rng.uniform(-5, 1, C_))).astype(np.float32)
+    tf = rng.uniform(-1, 1, C_).astype(np.float32)
+    ws_, refs = [], []
+    for _ in range(4):
+        w, r = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+        ws_.append(w)
+        refs.append(r)
+    ref = po.att_seq_v4_f16(x, sx, aa, bb, pp, ln_w, ln_b, *mixes, td, tf, *refs)
+    x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
+    ao, bo, po_ = (DevBuf.empty(C_, np.float32) for _ in range(3))
+    ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, 4 * C_))
+    fr.check(L().frhip_att_seq_v4(T, C_, keep(x).ptr, keep(sx).ptr, keep(aa).ptr, keep(bb).ptr, keep(pp).ptr,
+                                  keep(ln_w).ptr, keep(ln_b).ptr, *[keep(m).ptr for m in mixes], keep(td).ptr,
+                                  keep(tf).ptr, *[w.ref for w in ws_], x_out.ptr, xx_out.ptr, ao.ptr, bo.ptr, po_.ptr,
+                                  ws.ptr, None))
+    assert_close_f16(xx_out.numpy(), ref[1], max_ulp=1, what="xx_last")
+    assert_close_f16(x_out.numpy(), ref[0], max_ulp=3, max_frac=0.1, what="x_out")
+    # the carried state: same value, possibly another exponent offset pp -> compare aa*e^pp etc.
+    for got, want in ((ao, ref[2]), (bo, ref[3])):
+        g = got.numpy().astype(np.float64) * np.exp(po_.numpy().astype(np.float64) - ref[4].astype(np.float64))
+        assert np.allclose(g, want, rtol=2e-3, atol=2e-3 * np.abs(want).max())
+    assert np.abs(po_.numpy() - ref[4]).max() < 30  # offsets stay in a sane range
+
+
+@pytest.mark.parametrize("T,C_,H_", [(48, 512, 8), (512, 2560, 40), (1, 512, 8), (77, 512, 8)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_att_seq_v5_2(T, C_, H_, quant):
+    if C_ == 2560 and quant:
+        pytest.skip("full-size case runs once")
+    S_ = C_ // H_
+    x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
+    s = rng.standard_normal((H_, S_, S_)).astype(np.float32)
+    ln_w, ln_b = _common(C_)
+    lx_w = (1 + 0.1 * rng.standard_normal(C_)).astype(np.float32)
+    lx_b = (0.1 * rng.standard_normal(C_)).astype(np.float32)
+    mixes = [h(rng.uniform(0, 1, C_)) for _ in range(4)]
+    td = np.exp(-np.exp(rng.uniform(-6, 0, (H_, S_)))).astype(np.float32)
+    tf = rng.uniform(-1, 1, (H_, S_)).astype(np.float32)
+    ws_, refs = [], []
+    for _ in range(5):
+        w, r = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+        ws_.append(w)
+        refs.append(r)
+    ref_x, ref_xx, ref_s = po.att_v5_2_f16(x if T > 1 else x[0], sx, s, ln_w, ln_b, lx_w, lx_b, *mixes, td, tf, *refs, H_)
+    x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
+    s_out = DevBuf.empty((H_, S_, S_), np.float32)
+    ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, 4 * C_))
+    fr.check(L().frhip_att_seq_v5_2(T, C_, H_, keep(x).ptr, keep(sx).ptr, keep(s).ptr, keep(ln_w).ptr, keep(ln_b).ptr,
+                                    keep(lx_w).ptr, keep(lx_b).ptr, *[keep(m).ptr for m in mixes], keep(td).ptr,
+                                    keep(tf).ptr, *[w.ref for w in ws_], x_out.ptr, xx_out.ptr, s_out.ptr, ws.ptr,
+                                    None))
+    assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx_last")
+    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-4, atol=1e-4 * np.abs(ref_s).max())
+    assert_close_f16(x_out.numpy().reshape(ref_x.shape), ref_x, max_ulp=4, max_frac=0.2, what="x_out", floor_rms=1.0)
