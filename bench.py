@@ -134,6 +134,53 @@ def measure_kernels(fr, cfg, reps=20):
     return ms.value / reps, n_launch
 
 
+def probe_bandwidth(fr, nbytes=2 << 30, reps=5):
+    """Read-only and copy ceilings of this GPU as seen by plain streaming kernels (GB/s)."""
+    lib = fr.lib()
+    fr.init()
+    src, dst = fr.DevBuf(nbytes), fr.DevBuf(nbytes)
+    sink = fr.DevBuf(1 << 16)
+    fr.check(lib.frhip_memset_async(src.ptr, 1, nbytes, None))
+    st = C.c_void_p()
+    fr.check(lib.frhip_stream_create(C.byref(st)))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.frhip_event_create(C.byref(e0))
+    lib.frhip_event_create(C.byref(e1))
+    out = {}
+    for name, fn, traffic in (("read", lambda: lib.frhip_read_probe(src.ptr, nbytes, sink.ptr, st), nbytes),
+                              ("copy", lambda: lib.frhip_copy_probe(dst.ptr, src.ptr, nbytes, st), 2 * nbytes)):
+        fr.check(fn())
+        fr.check(lib.frhip_stream_sync(st))
+        fr.check(lib.frhip_event_record(e0, st))
+        for _ in range(reps):
+            fr.check(fn())
+        fr.check(lib.frhip_event_record(e1, st))
+        fr.check(lib.frhip_event_sync(e1))
+        ms = C.c_float()
+        fr.check(lib.frhip_event_elapsed_ms(e0, e1, C.byref(ms)))
+        out[name + "_GBs"] = round(traffic * reps / (ms.value * 1e-3) / 1e9, 1)
+    lib.frhip_stream_destroy(st)
+    return out
+
+
+def prefill_extra(fr):
+    """BASELINE configuration 4: T=1024 seq-mode prefill of the same fp16 model."""
+    cfg = CONFIGS["fp16"]
+    m = fr.Model(cfg["spec"], cfg["strategy"])
+    ids = np.random.default_rng(43).integers(0, V_, 1024)
+    best = 1e9
+    for _ in range(4):
+        m.reset()
+        t0 = time.perf_counter()
+        m.run(ids)
+        best = min(best, time.perf_counter() - t0)
+    m.close()
+    flops = 2.0 * 1024 * L_ * 54525952
+    return {"prefill_T1024_tok_s": round(1024 / best, 1), "prefill_ms": round(best * 1e3, 3),
+            "prefill_gemm_TFLOPs_over_whole_pass": round(flops / best / 1e12, 1),
+            "prefill_frac_of_2500_TFLOPs": round(flops / best / 2.5e15, 4)}
+
+
 def cpu_baseline(seconds_budget=20.0):
     """The oracle's fp32 one-token forward on the host cores (OpenMP over output columns), on
     the same architecture with the depth cut to 2 layers + head to bound the run; the
@@ -187,6 +234,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--dtype", choices=["fp16", "int8"], default="fp16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the int8-decode and prefill side measurements")
+    ap.add_argument("--probe", action="store_true", help="only run the read/copy bandwidth probes and print them")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs batch-1 decode on ONE GPU; --gpus %d is not supported "
@@ -195,6 +244,9 @@ def main():
         sys.exit("bench.py: launched with WORLD_SIZE > 1; only a single rank is supported")
 
     fr = importlib.import_module("faster-rwkv_amd")
+    if args.probe:
+        print(json.dumps(probe_bandwidth(fr)), flush=True)
+        return
     cfg = CONFIGS[args.dtype]
     t0 = time.perf_counter()
     model = fr.Model(cfg["spec"], cfg["strategy"])
@@ -228,10 +280,23 @@ def main():
                      "avg_launch_us": round(1e3 * kernel_ms / n_launch, 3)},
         "roofline_tok_s": round(1.0 / (abytes / (HBM_PEAK_GBS * 1e9)), 1),
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
-    else:
-        out["cpu_baseline"] = None
+    if not args.no_extras:
+        extra = {}
+        other = "int8" if args.dtype == "fp16" else "fp16"
+        ocfg = CONFIGS[other]
+        om = fr.Model(ocfg["spec"], ocfg["strategy"])
+        om.greedy(0, args.warmup)
+        _, osecs = om.greedy(17, args.steps)
+        om.close()
+        okms, _ = measure_kernels(fr, ocfg)
+        ob = algorithmic_bytes_per_token(ocfg["wbytes"])
+        extra[other + "_decode_tok_s"] = round(args.steps / osecs, 2)
+        extra[other + "_gemv_GBs"] = round(ob / (okms * 1e-3) / 1e9, 1)
+        extra[other + "_gemv_frac_of_hbm_peak"] = round(ob / (okms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        extra.update(prefill_extra(fr))
+        extra.update(probe_bandwidth(fr))
+        out["extra"] = extra
+    out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()
     print(json.dumps(out), flush=True)
 
 

@@ -89,6 +89,8 @@ _SIGS = {
     "frhip_att_one_v5_1": (_i, [_i, _i] + [_vp] * 13 + [_WP] * 5 + [_vp] * 5),
     "frhip_argmax_f32": (_i, [_vp, _i, _vp, _vp]),
     "frhip_gemm": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
+    "frhip_copy_probe": (_i, [_vp, _vp, _sz, _vp]),
+    "frhip_read_probe": (_i, [_vp, _sz, _vp, _vp]),
     "frhip_seq_workspace_bytes": (_sz, [_i, _i, _i]),
     "frhip_ffn_seq": (_i, [_i, _i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
     "frhip_att_seq_v4": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),

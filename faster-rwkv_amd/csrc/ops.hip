@@ -143,6 +143,25 @@ __global__ void dequant_u8_kernel(const uint32_t* __restrict__ q, const h1* __re
   out[i] = (h4){lo.x, lo.y, hi.x, hi.y};
 }
 
+__global__ __launch_bounds__(256) void copy_probe_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+__global__ __launch_bounds__(512) void read_probe_kernel(const u32x4* __restrict__ src, size_t n, uint32_t* sink) {
+  u32x4 acc = {0, 0, 0, 0};
+  const size_t stride = (size_t)gridDim.x * 512;
+  size_t i = (size_t)blockIdx.x * 512 + threadIdx.x;
+  for (; i + 3 * stride < n; i += 4 * stride) {
+    u32x4 a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride);
+    u32x4 c = __builtin_nontemporal_load(src + i + 2 * stride), d = __builtin_nontemporal_load(src + i + 3 * stride);
+    acc ^= a ^ b ^ c ^ d;
+  }
+  for (; i < n; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  uint32_t v = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off);
+  if ((threadIdx.x & 63) == 0 && threadIdx.x == 0) sink[blockIdx.x] = v;
+}
+
 // Index of the maximum, first occurrence on ties; single workgroup of 1024 threads.
 __global__ __launch_bounds__(1024) void argmax_f32_kernel(const float* __restrict__ x, int n, int32_t* out) {
   __shared__ float bv[16];
@@ -296,6 +315,26 @@ int frhip_dequant_u8(const frhip_weight* w, void* dst, frhip_stream s) {
                      (const uint32_t*)w->data, (const h1*)w->mx, (const h1*)w->rx, (const h1*)w->my, (const h1*)w->ry,
                      (h4*)dst, w->K, w->N);
   return check_launch("dequant_u8");
+}
+
+int frhip_copy_probe(void* dst, const void* src, size_t bytes, frhip_stream s) {
+  if (!dst || !src) return set_error(FRHIP_EINVAL, "copy_probe: null pointer");
+  if (bytes % 16 != 0) return set_error(FRHIP_ESHAPE, "copy_probe: bytes must be a multiple of 16");
+  if (bytes == 0) return 0;
+  hipLaunchKernelGGL(copy_probe_kernel, dim3(compute_units() * 8), dim3(256), 0, static_cast<hipStream_t>(s),
+                     (const u32x4*)src, (u32x4*)dst, bytes / 16);
+  return check_launch("copy_probe");
+}
+
+int frhip_read_probe(const void* src, size_t bytes, void* sink, frhip_stream s) {
+  if (!src || !sink) return set_error(FRHIP_EINVAL, "read_probe: null pointer");
+  if (bytes % 16 != 0) return set_error(FRHIP_ESHAPE, "read_probe: bytes must be a multiple of 16");
+  if (bytes == 0) return 0;
+  int grid = compute_units() * 2;
+  if (grid > 2048) grid = 2048;
+  hipLaunchKernelGGL(read_probe_kernel, dim3(grid), dim3(512), 0, static_cast<hipStream_t>(s), (const u32x4*)src,
+                     bytes / 16, (uint32_t*)sink);
+  return check_launch("read_probe");
 }
 
 int frhip_argmax_f32(const float* logits, int n, int32_t* out_id, frhip_stream s) {

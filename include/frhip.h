@@ -198,6 +198,15 @@ int frhip_att_seq_v5_2(int T, int C, int H, const void *x, const void *sx, const
                        const frhip_weight *gw, const frhip_weight *ow,
                        void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
 
+/* ---- bandwidth probes (measurement aids, no counterpart in the reference) --------- */
+/* Plain device copy, 16 bytes per lane: the kernel of known traffic (bytes read + bytes
+ * written) against which hardware counters are scaled. */
+int frhip_copy_probe(void *dst, const void *src, size_t bytes, frhip_stream s);
+/* Streams `bytes` of device memory once through the wavefronts (non-temporal 16-byte loads,
+ * xor-folded so the loads are not dead) and writes one word per workgroup to `sink`
+ * (at least 8192 bytes): the read-only ceiling the row-streaming kernels are compared with. */
+int frhip_read_probe(const void *src, size_t bytes, void *sink, frhip_stream s);
+
 /* greedy sampler step (Sampler::Sample with top_k = 1, chat.cpp:76-77): index of the
  * largest logit, first one on ties, written to *out_id on the device. */
 int frhip_argmax_f32(const float *logits, int n, int32_t *out_id, frhip_stream s);
