@@ -23,6 +23,7 @@
 // One RWKV-4 layer is four launches; the reference issues seventeen
 // (kernels/cuda/att.cu:182-217, ffn.cu:62-87).
 #include <climits>
+#include <cstdlib>
 #include <cstring>
 #include <type_traits>
 
@@ -594,7 +595,16 @@ static int round_nch(int nch) {
 // Rows in flight per wave.  When all rows of a wave fit in kMaxLoads loads per lane they
 // form one batch (multi = false); otherwise batches of at most kMaxLoads/2 loads alternate
 // between two register sets.
-static int pick_r(const RowsArgs& a, int grid, int nch, bool* multi) {
+static int env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return (e && atoi(e) > 0) ? atoi(e) : dflt;
+}
+
+static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
+  // uint8 rows cost several VALU operations per element: smaller batches let the dequantisation
+  // of one batch overlap the loads of the next
+  static const int max_u8 = env_int("FRHIP_MAXLOADS_U8", kMaxLoads);
+  const int kMaxLoads = u8 ? max_u8 : frhip::kMaxLoads;
   const long waves = (long)grid * kWaves;
   long per = ((long)a.start[a.nseg] + waves - 1) / waves;  // most rows any wave gets
   if (per < 1) per = 1;
@@ -653,7 +663,7 @@ static int launch_rows(const RowsArgs& a, bool u8, hipStream_t st, const char* w
   if (nch < 0) return set_error(FRHIP_ESHAPE, "K is too large for the row-streaming kernel (max 9216 fp16 / 18432 uint8)");
   const int grid = decode_grid();
   bool multi = false;
-  const int R = pick_r(a, grid, nch, &multi);
+  const int R = pick_r(a, grid, nch, u8, &multi);
   const size_t lds = 2 * (size_t)a.K * (a.nvec + (u8 ? 2 * a.nseg : 0));
   FR_TRY(check_lds(lds));
   bool ok = false;

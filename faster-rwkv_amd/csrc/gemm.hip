@@ -4,8 +4,8 @@
 //
 // Both operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
 // a lane's A (or B) fragment is 8 consecutive k of one row, i.e. one 16-byte load.
-// Workgroup tile 128x128, K step 64, 256 threads = 2x2 waves of 64x64 (2x2 MFMA tiles,
-// 64 fp32 accumulators per lane).  Tiles of X and Wt go global -> registers -> LDS
+// Workgroup tile 128x128 (64x128 for launches that would otherwise leave CUs idle), K step 64,
+// 256 threads = 2x2 waves of 64x64 (2x2 MFMA tiles, 64 fp32 accumulators per lane).  Tiles of X and Wt go global -> registers -> LDS
 // (rows padded by 16 bytes against bank conflicts); the loads of step k+1 are issued
 // before the MFMAs of step k.  uint8 weights are dequantised to binary16 on their way
 // into LDS with the same formula as the one-token kernels, so the product sees exactly
@@ -24,10 +24,14 @@ namespace frhip {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BK = 64, LDSK = BK + 8;
+constexpr int BN = 128, BK = 64, LDSK = BK + 8;
 constexpr int kGemmThreads = 256;
-template <bool U8>
+// BM = 128 (waves 2 x 2 of 64 x 64) or 64 (waves of 32 x 64), for launches that would otherwise
+// leave compute units idle.
+template <int BM, bool U8>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
+  constexpr int MI = BM / 64;   // 32-row MFMA blocks per wave
+  constexpr int AC = BM / 32;   // 16-byte chunks of the A tile per thread
   __shared__ __attribute__((aligned(16))) h1 As[BM][LDSK];
   __shared__ __attribute__((aligned(16))) h1 Bs[BN][LDSK];
 
@@ -47,12 +51,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
   // global -> register staging: a tile is 128 rows x 64 k.
   //   A (binary16): 1024 chunks of 8 halves, 4 per thread: chunk c -> row c/8, k (c%8)*8
   //   B binary16: same.  B uint8: 512 chunks of 16 codes, 2 per thread: row c/4, k (c%4)*16
-  h8 ra[4];
+  h8 ra[AC];
   h8 rb[4];
   u32x4 rq[2];
   auto load_tiles = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < AC; i++) {
       const int c = tid + i * kGemmThreads;
       int row = m0 + (c >> 3);
       row = row < M ? row : M - 1;  // rows past M are computed on a copy of the last row and never stored
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
   };
   auto store_tiles = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < AC; i++) {
       const int c = tid + i * kGemmThreads;
       *reinterpret_cast<h8*>(&As[c >> 3][(c & 7) * 8]) = ra[i];
     }
@@ -115,9 +119,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
     }
   };
 
-  f16v acc[2][2];
+  f16v acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < MI; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -131,14 +135,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
     if (k0 + BK < K) load_tiles(k0 + BK);
 #pragma unroll
     for (int ks = 0; ks < BK; ks += 16) {
-      h8 fa[2], fb[2];
+      h8 fa[MI], fb[2];
       const int kofs = ks + (lane >> 5) * 8;
 #pragma unroll
-      for (int i = 0; i < 2; i++) fa[i] = *reinterpret_cast<const h8*>(&As[wm * 64 + i * 32 + (lane & 31)][kofs]);
+      for (int i = 0; i < MI; i++) fa[i] = *reinterpret_cast<const h8*>(&As[wm * (BM / 2) + i * 32 + (lane & 31)][kofs]);
 #pragma unroll
       for (int j = 0; j < 2; j++) fb[j] = *reinterpret_cast<const h8*>(&Bs[wn * 64 + j * 32 + (lane & 31)][kofs]);
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
@@ -147,13 +151,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
 
   // epilogue: acc[i][j][v] is C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the 32x32 tile
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < MI; i++) {
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const int col = n0 + wn * 64 + j * 32 + (lane & 31);
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
         if (row < M && col < N) {
           const float s = acc[i][j][v];
           const size_t o = (size_t)row * N + col;
@@ -192,11 +196,21 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what) {
   }
   for (int s = a.nseg; s <= kGemmMaxSeg; s++) a.tile_start[s] = INT_MAX;
   a.tile_start[a.nseg] = tiles;
-  dim3 grid(tiles, (a.M + BM - 1) / BM);
-  if (u8)
-    hipLaunchKernelGGL(gemm_kernel<true>, grid, dim3(kGemmThreads), 0, st, a);
-  else
-    hipLaunchKernelGGL(gemm_kernel<false>, grid, dim3(kGemmThreads), 0, st, a);
+  // 128-row tiles unless that leaves fewer than ~1.5 workgroups per CU; then 64-row tiles
+  const int m128 = (a.M + 127) / 128;
+  if ((long)tiles * m128 < (long)compute_units() * 3 / 2) {
+    dim3 grid(tiles, (a.M + 63) / 64);
+    if (u8)
+      hipLaunchKernelGGL((gemm_kernel<64, true>), grid, dim3(kGemmThreads), 0, st, a);
+    else
+      hipLaunchKernelGGL((gemm_kernel<64, false>), grid, dim3(kGemmThreads), 0, st, a);
+  } else {
+    dim3 grid(tiles, m128);
+    if (u8)
+      hipLaunchKernelGGL((gemm_kernel<128, true>), grid, dim3(kGemmThreads), 0, st, a);
+    else
+      hipLaunchKernelGGL((gemm_kernel<128, false>), grid, dim3(kGemmThreads), 0, st, a);
+  }
   return check_launch(what);
 }
 
