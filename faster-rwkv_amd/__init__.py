@@ -87,6 +87,7 @@ _SIGS = {
     "frhip_ffn_one": (_i, [_i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
     "frhip_head": (_i, [_i, _vp, _vp, _vp, _WP, _vp, _vp]),
     "frhip_att_one_v5_1": (_i, [_i, _i] + [_vp] * 13 + [_WP] * 5 + [_vp] * 5),
+    "frhip_att_one_v5": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 5),
     "frhip_argmax_f32": (_i, [_vp, _i, _vp, _vp]),
     "frhip_gemm": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
     "frhip_copy_probe": (_i, [_vp, _vp, _sz, _vp]),
@@ -95,6 +96,7 @@ _SIGS = {
     "frhip_ffn_seq": (_i, [_i, _i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
     "frhip_att_seq_v4": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),
     "frhip_att_seq_v5_2": (_i, [_i, _i, _i] + [_vp] * 13 + [_WP] * 5 + [_vp] * 5),
+    "frhip_att_seq_v5": (_i, [_i, _i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 5),
 }
 
 _lib = None
@@ -238,6 +240,8 @@ def host():
         h.fr_model_free.argtypes = [_vp]
         h.fr_model_info.argtypes = [_vp, C.POINTER(_i)]
         h.fr_model_run.argtypes = [_vp, _vp, _i, _vp, _i]
+        h.fr_model_run_full.restype = C.c_longlong
+        h.fr_model_run_full.argtypes = [_vp, _vp, _i, _vp, C.c_longlong]
         h.fr_model_reset.argtypes = [_vp]
         h.fr_model_save_state.argtypes = [_vp, C.c_char_p]
         h.fr_model_load_state.argtypes = [_vp, C.c_char_p]
@@ -275,6 +279,13 @@ class Model:
         n = self._chk(self._h.fr_model_run(self._m, ids.ctypes.data, len(ids), self._logits.ctypes.data,
                                            self._logits.size))
         return self._logits[:n].copy()
+
+    def run_full(self, ids):
+        """ModelForwardSeq(..., full_output=true): fp32 logits of every position, [T, vocab]."""
+        ids = np.ascontiguousarray(ids, np.int32)
+        out = np.empty((len(ids), self._logits.size), np.float32)
+        n = self._chk(self._h.fr_model_run_full(self._m, ids.ctypes.data, len(ids), out.ctypes.data, out.size))
+        return out.reshape(-1)[:n].reshape(len(ids), -1)
 
     def reset(self):
         self._chk(self._h.fr_model_reset(self._m))

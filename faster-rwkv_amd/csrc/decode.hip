@@ -480,8 +480,9 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
 // ===========================================================================
 struct Wkv5One {
   int H;
+  int uw_head;  // 0: u, w are [H][S] (RWKV-5.1/5.2); 1: one value per head (RWKV-5.0)
   const float *s, *r, *k, *v, *w, *u, *lx_w, *lx_b;
-  const h1* g;
+  const h1* g;  // gate, or null (RWKV-5.0 has none)
   float* s_out;
   h1* gated_out;
 };
@@ -497,8 +498,8 @@ __global__ __launch_bounds__(256) void wkv5_one_kernel(Wkv5One a) {
     rk[0][t] = a.r[h * S + t];
     rk[1][t] = a.k[h * S + t];
     rk[2][t] = a.v[h * S + t];
-    uw[0][t] = a.u[h * S + t];
-    uw[1][t] = a.w[h * S + t];
+    uw[0][t] = a.u[a.uw_head ? h : h * S + t];
+    uw[1][t] = a.w[a.uw_head ? h : h * S + t];
   }
   const float* sh = a.s + (size_t)h * S * S;
   float* so = a.s_out + (size_t)h * S * S;
@@ -529,7 +530,7 @@ __global__ __launch_bounds__(256) void wkv5_one_kernel(Wkv5One a) {
     const float inv = 1.0f / sqrtf(var + 1e-5f);
     const int c = h * S + t;
     const float y = d * inv * a.lx_w[c] + a.lx_b[c];
-    a.gated_out[c] = (h1)y * a.g[c];
+    a.gated_out[c] = a.g ? (h1)y * a.g[c] : (h1)y;
   }
 }
 
@@ -807,14 +808,15 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_out");
 }
 
-extern "C" int frhip_att_one_v5_1(int C, int H, const void* x, const void* sx, const float* s, const void* ln_w,
+// Shared by RWKV-5.0 (no gate: g_mix and gw null, u and w per head) and RWKV-5.1/5.2.
+static int att_one_v5_impl(bool v50, int C, int H, const void* x, const void* sx, const float* s, const void* ln_w,
                                   const void* ln_b, const float* lx_w, const float* lx_b, const void* k_mix,
                                   const void* v_mix, const void* r_mix, const void* g_mix, const float* t_decay,
                                   const float* t_first, const frhip_weight* kw, const frhip_weight* vw,
                                   const frhip_weight* rw, const frhip_weight* gw, const frhip_weight* ow,
                                   void* x_out, void* xx_out, float* s_out, void* workspace, frhip_stream s_) {
   FR_TRY(check_embd(C));
-  if (H <= 0 || C % H != 0 || C / H != 64) return set_error(FRHIP_ESHAPE, "att_one_v5_1: head size must be 64");
+  if (H <= 0 || C % H != 0 || C / H != 64) return set_error(FRHIP_ESHAPE, "att_one_v5: head size must be 64");
   FR_TRY(check_vec(x, "x is null or misaligned"));
   FR_TRY(check_vec(sx, "sx is null or misaligned"));
   FR_TRY(check_vec(ln_w, "ln_w is null or misaligned"));
@@ -822,39 +824,40 @@ extern "C" int frhip_att_one_v5_1(int C, int H, const void* x, const void* sx, c
   FR_TRY(check_vec(k_mix, "k_mix is null or misaligned"));
   FR_TRY(check_vec(v_mix, "v_mix is null or misaligned"));
   FR_TRY(check_vec(r_mix, "r_mix is null or misaligned"));
-  FR_TRY(check_vec(g_mix, "g_mix is null or misaligned"));
+  if (!v50) FR_TRY(check_vec(g_mix, "g_mix is null or misaligned"));
   FR_TRY(check_vec(x_out, "x_out is null or misaligned"));
   FR_TRY(check_vec(xx_out, "xx_out is null or misaligned"));
   FR_TRY(check_vec(workspace, "workspace is null or misaligned"));
-  if (!s || !s_out || !lx_w || !lx_b || !t_decay || !t_first) return set_error(FRHIP_EINVAL, "att_one_v5_1: null state or parameter");
-  if (xx_out == sx) return set_error(FRHIP_EINVAL, "att_one_v5_1: xx_out must not alias sx");
+  if (!s || !s_out || !lx_w || !lx_b || !t_decay || !t_first) return set_error(FRHIP_EINVAL, "att_one_v5: null state or parameter");
+  if (xx_out == sx) return set_error(FRHIP_EINVAL, "att_one_v5: xx_out must not alias sx");
   FR_TRY(check_weight(kw, C, C));
   FR_TRY(check_weight(vw, C, C));
   FR_TRY(check_weight(rw, C, C));
-  FR_TRY(check_weight(gw, C, C));
+  if (!v50) FR_TRY(check_weight(gw, C, C));
   FR_TRY(check_weight(ow, C, C));
-  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype || kw->dtype != gw->dtype)
-    return set_error(FRHIP_EINVAL, "att_one_v5_1: key/value/receptance/gate dtypes differ");
+  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype || (!v50 && kw->dtype != gw->dtype))
+    return set_error(FRHIP_EINVAL, "att_one_v5: key/value/receptance/gate dtypes differ");
   hipStream_t st = static_cast<hipStream_t>(s_);
   Workspace w = carve(workspace, C);
 
   // LN -> 4 mixes -> k, v, r (fp32) and g = silu(.) (half)      att.cu:276-290
   RowsArgs a = empty_args(C);
   a.prologue = P_LN_MIX;
-  a.nvec = 4;
+  a.nvec = v50 ? 3 : 4;
   a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
   a.mix[0] = (const h1*)k_mix; a.mix[1] = (const h1*)v_mix; a.mix[2] = (const h1*)r_mix; a.mix[3] = (const h1*)g_mix;
   a.xx_out = (h1*)xx_out;
   add_seg(a, kw, 0, E_STORE_F32, w.k32);
   add_seg(a, vw, 1, E_STORE_F32, w.v32);
   add_seg(a, rw, 2, E_STORE_F32, w.r32);
-  add_seg(a, gw, 3, E_SILU, w.g);
+  if (!v50) add_seg(a, gw, 3, E_SILU, w.g);
   FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "att_v5_front"));
 
   Wkv5One k;
   k.H = H;
+  k.uw_head = v50 ? 1 : 0;
   k.s = s; k.r = w.r32; k.k = w.k32; k.v = w.v32; k.w = t_decay; k.u = t_first; k.lx_w = lx_w; k.lx_b = lx_b;
-  k.g = w.g; k.s_out = s_out; k.gated_out = w.rwkv;
+  k.g = v50 ? nullptr : w.g; k.s_out = s_out; k.gated_out = w.rwkv;
   hipLaunchKernelGGL(wkv5_one_kernel, dim3(H), dim3(256), 0, st, k);
   FR_TRY(check_launch("wkv5_one"));
 
@@ -865,6 +868,27 @@ extern "C" int frhip_att_one_v5_1(int C, int H, const void* x, const void* sx, c
   b.res_x = (const h1*)x;
   add_seg(b, ow, 0, E_RESIDUAL, x_out);
   return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_v5_out");
+}
+
+extern "C" int frhip_att_one_v5_1(int C, int H, const void* x, const void* sx, const float* s, const void* ln_w,
+                                  const void* ln_b, const float* lx_w, const float* lx_b, const void* k_mix,
+                                  const void* v_mix, const void* r_mix, const void* g_mix, const float* t_decay,
+                                  const float* t_first, const frhip_weight* kw, const frhip_weight* vw,
+                                  const frhip_weight* rw, const frhip_weight* gw, const frhip_weight* ow,
+                                  void* x_out, void* xx_out, float* s_out, void* workspace, frhip_stream s_) {
+  return att_one_v5_impl(false, C, H, x, sx, s, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, g_mix, t_decay, t_first,
+                         kw, vw, rw, gw, ow, x_out, xx_out, s_out, workspace, s_);
+}
+
+// att_one_v5 (RWKV-5.0): kernels/cuda/att.cu:219-265,362-391.
+extern "C" int frhip_att_one_v5(int C, int H, const void* x, const void* sx, const float* s, const void* ln_w,
+                                const void* ln_b, const float* lx_w, const float* lx_b, const void* k_mix,
+                                const void* v_mix, const void* r_mix, const float* t_decay, const float* t_first,
+                                const frhip_weight* kw, const frhip_weight* vw, const frhip_weight* rw,
+                                const frhip_weight* ow, void* x_out, void* xx_out, float* s_out, void* workspace,
+                                frhip_stream s_) {
+  return att_one_v5_impl(true, C, H, x, sx, s, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, nullptr, t_decay, t_first,
+                         kw, vw, rw, nullptr, ow, x_out, xx_out, s_out, workspace, s_);
 }
 
 extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const void* ln_w, const void* ln_b,

@@ -170,8 +170,9 @@ __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
 // ---------------------------------------------------------------------------
 struct Wkv5Seq {
   int T, C, H, Lc, nchunk;
+  int uw_head;       // 0: u, w are [H][64] (RWKV-5.2); 1: one value per head (RWKV-5.0)
   const float *r, *k, *v, *w, *u, *lx_w, *lx_b;
-  const h1* g;       // [T][C] gate, already through silu
+  const h1* g;       // [T][C] gate, already through silu; null for RWKV-5.0
   const float* s;    // state before the sequence
   float* loc;        // [nchunk][H][64][64] local end states
   float* sin;        // [nchunk][H][64][64] state at the start of each chunk
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(256) void wkv5_local_kernel(Wkv5Seq a) {
     kk[e] = a.k[src];
     vv[e] = a.v[src];
   }
-  if (t < S5) wsh[t] = a.w[h * S5 + t];
+  if (t < S5) wsh[t] = a.w[a.uw_head ? h : h * S5 + t];
   __syncthreads();
   float s[16];
 #pragma unroll
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(256) void wkv5_carry_kernel(Wkv5Seq a) {
   const size_t per = (size_t)a.H * S5 * S5;
   if (e >= per) return;
   const int i = (int)((e / S5) % S5), h = (int)(e / (S5 * S5));
-  const float w = a.w[h * S5 + i];
+  const float w = a.w[a.uw_head ? h : h * S5 + i];
   float s = a.s[e];
   for (int ch = 0; ch < a.nchunk; ch++) {
     a.sin[(size_t)ch * per + e] = s;
@@ -244,8 +245,8 @@ __global__ __launch_bounds__(256) void wkv5_apply_kernel(Wkv5Seq a) {
     vv[e] = a.v[src];
   }
   if (t < S5) {
-    wsh[t] = a.w[h * S5 + t];
-    ush[t] = a.u[h * S5 + t];
+    wsh[t] = a.w[a.uw_head ? h : h * S5 + t];
+    ush[t] = a.u[a.uw_head ? h : h * S5 + t];
   }
   const float* src = a.sin + ((size_t)ch * a.H + h) * S5 * S5;
   float s[16];
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(256) void wkv5_apply_kernel(Wkv5Seq a) {
       const float inv = 1.0f / sqrtf(var + 1e-5f);
       const float y = d * inv * gw + gb;
       const size_t oi = (size_t)(t0 + tt) * a.C + h * S5 + t;
-      a.gated[oi] = (h1)y * a.g[oi];
+      a.gated[oi] = a.g ? (h1)y * a.g[oi] : (h1)y;
     }
   }
   if (ch == a.nchunk - 1) {
@@ -464,46 +465,47 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v4 out");
 }
 
-// att_seq_v5_2 (kernels/cuda/att_seq.cu:368-423,464-493).
-extern "C" int frhip_att_seq_v5_2(int T, int C, int H, const void* x, const void* sx, const float* s_in,
+// Shared by RWKV-5.0 (no gate, u and w per head) and RWKV-5.2.
+static int att_seq_v5_impl(bool v50, int T, int C, int H, const void* x, const void* sx, const float* s_in,
                                   const void* ln_w, const void* ln_b, const float* lx_w, const float* lx_b,
                                   const void* k_mix, const void* v_mix, const void* r_mix, const void* g_mix,
                                   const float* t_decay, const float* t_first, const frhip_weight* kw,
                                   const frhip_weight* vw, const frhip_weight* rw, const frhip_weight* gw,
                                   const frhip_weight* ow, void* x_out, void* xx_out, float* s_out, void* workspace,
                                   frhip_stream s) {
-  if (T <= 0) return set_error(FRHIP_ESHAPE, "att_seq_v5_2: T must be positive");
-  if (!x || !sx || !s_in || !ln_w || !ln_b || !lx_w || !lx_b || !k_mix || !v_mix || !r_mix || !g_mix || !t_decay ||
+  if (T <= 0) return set_error(FRHIP_ESHAPE, "att_seq_v5: T must be positive");
+  if (!x || !sx || !s_in || !ln_w || !ln_b || !lx_w || !lx_b || !k_mix || !v_mix || !r_mix || (!v50 && !g_mix) || !t_decay ||
       !t_first || !x_out || !xx_out || !s_out || !workspace)
-    return set_error(FRHIP_EINVAL, "att_seq_v5_2: null pointer");
-  if (H <= 0 || C % H != 0 || C / H != 64) return set_error(FRHIP_ESHAPE, "att_seq_v5_2: head size must be 64");
-  FR_TRY(check_w(kw, C, C, "att_seq_v5_2: bad key weight"));
-  FR_TRY(check_w(vw, C, C, "att_seq_v5_2: bad value weight"));
-  FR_TRY(check_w(rw, C, C, "att_seq_v5_2: bad receptance weight"));
-  FR_TRY(check_w(gw, C, C, "att_seq_v5_2: bad gate weight"));
-  FR_TRY(check_w(ow, C, C, "att_seq_v5_2: bad output weight"));
-  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype || kw->dtype != gw->dtype)
-    return set_error(FRHIP_EINVAL, "att_seq_v5_2: k/v/r/g dtypes differ");
+    return set_error(FRHIP_EINVAL, "att_seq_v5: null pointer");
+  if (H <= 0 || C % H != 0 || C / H != 64) return set_error(FRHIP_ESHAPE, "att_seq_v5: head size must be 64");
+  FR_TRY(check_w(kw, C, C, "att_seq_v5: bad key weight"));
+  FR_TRY(check_w(vw, C, C, "att_seq_v5: bad value weight"));
+  FR_TRY(check_w(rw, C, C, "att_seq_v5: bad receptance weight"));
+  if (!v50) FR_TRY(check_w(gw, C, C, "att_seq_v5: bad gate weight"));
+  FR_TRY(check_w(ow, C, C, "att_seq_v5: bad output weight"));
+  if (kw->dtype != vw->dtype || kw->dtype != rw->dtype || (!v50 && kw->dtype != gw->dtype))
+    return set_error(FRHIP_EINVAL, "att_seq_v5: k/v/r/g dtypes differ");
   hipStream_t st = static_cast<hipStream_t>(s);
   SeqWs w = carve_seq(workspace, T, C, 64);
   const void* mixes[4] = {k_mix, v_mix, r_mix, g_mix};
   h1* outs[4] = {w.m0, w.m1, w.m2, w.m3};
-  FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, 4, xx_out, st));
+  FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, v50 ? 3 : 4, xx_out, st));
   GemmArgs a;
   memset(&a, 0, sizeof(a));
   a.M = T; a.K = C;
   gemm_add_seg(a, w.m0, kw, w.f0, G_STORE_F32);  // k
   gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
   gemm_add_seg(a, w.m2, rw, w.f2, G_STORE_F32);  // r
-  gemm_add_seg(a, w.m3, gw, w.g, G_SILU);        // g
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5_2 k,v,r,g"));
+  if (!v50) gemm_add_seg(a, w.m3, gw, w.g, G_SILU);  // g
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5 k,v,r,g"));
 
   Wkv5Seq q;
   q.T = T; q.C = C; q.H = H;
+  q.uw_head = v50 ? 1 : 0;
   q.Lc = pick_chunk(T, H);
   q.nchunk = (T + q.Lc - 1) / q.Lc;
   q.r = w.f2; q.k = w.f0; q.v = w.f1; q.w = t_decay; q.u = t_first; q.lx_w = lx_w; q.lx_b = lx_b;
-  q.g = w.g; q.s = s_in; q.s_out = s_out; q.gated = w.gated;
+  q.g = v50 ? nullptr : w.g; q.s = s_in; q.s_out = s_out; q.gated = w.gated;
   const size_t per = al256(4 * (size_t)q.nchunk * C * 64) / 4;
   q.loc = w.scan;
   q.sin = q.loc + per;
@@ -518,5 +520,30 @@ extern "C" int frhip_att_seq_v5_2(int T, int C, int H, const void* x, const void
   b.M = T; b.K = C;
   b.res_x = (const h1*)x;
   gemm_add_seg(b, w.gated, ow, x_out, G_RESIDUAL);
-  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5_2 out");
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5 out");
+}
+
+// att_seq_v5_2 (kernels/cuda/att_seq.cu:368-423,464-493).
+extern "C" int frhip_att_seq_v5_2(int T, int C, int H, const void* x, const void* sx, const float* s_in,
+                                  const void* ln_w, const void* ln_b, const float* lx_w, const float* lx_b,
+                                  const void* k_mix, const void* v_mix, const void* r_mix, const void* g_mix,
+                                  const float* t_decay, const float* t_first, const frhip_weight* kw,
+                                  const frhip_weight* vw, const frhip_weight* rw, const frhip_weight* gw,
+                                  const frhip_weight* ow, void* x_out, void* xx_out, float* s_out, void* workspace,
+                                  frhip_stream s) {
+  return att_seq_v5_impl(false, T, C, H, x, sx, s_in, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, g_mix, t_decay,
+                         t_first, kw, vw, rw, gw, ow, x_out, xx_out, s_out, workspace, s);
+}
+
+// att_seq_v5 (RWKV-5.0): kernels/cuda/att_seq.cu:158-256,425-462.  The reference evaluates the
+// recurrence in matrix form (decay powers times r k^T, att_seq.cu:181-243); here the same sums
+// are taken by the chunked scan that serves RWKV-5.2, with u and w constant over a head.
+extern "C" int frhip_att_seq_v5(int T, int C, int H, const void* x, const void* sx, const float* s_in,
+                                const void* ln_w, const void* ln_b, const float* lx_w, const float* lx_b,
+                                const void* k_mix, const void* v_mix, const void* r_mix, const float* t_decay,
+                                const float* t_first, const frhip_weight* kw, const frhip_weight* vw,
+                                const frhip_weight* rw, const frhip_weight* ow, void* x_out, void* xx_out,
+                                float* s_out, void* workspace, frhip_stream s) {
+  return att_seq_v5_impl(true, T, C, H, x, sx, s_in, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, nullptr, t_decay,
+                         t_first, kw, vw, rw, nullptr, ow, x_out, xx_out, s_out, workspace, s);
 }

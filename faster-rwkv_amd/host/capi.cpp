@@ -16,7 +16,7 @@ void allocator_stats(size_t *reserved, size_t *in_use, size_t *driver_calls);
 
 namespace {
 thread_local std::string g_err;
-template <typename F> int guarded(F &&f) {
+template <typename F> auto guarded(F &&f) -> decltype(f()) {
   try {
     return f();
   } catch (const std::exception &e) {
@@ -76,6 +76,20 @@ int fr_model_run(void *m, const int *ids, int n, float *logits, int capacity) {
     auto *model = static_cast<rwkv::Model *>(m);
     rwkv::Tensor out = n == 1 ? model->Run(ids[0]) : model->Run(std::vector<int>(ids, ids + n));
     const int v = static_cast<int>(out.numel());
+    if (v > capacity) throw FRException("logits buffer too small");
+    std::memcpy(logits, out.data_ptr<float>(), sizeof(float) * static_cast<size_t>(v));
+    return v;
+  });
+}
+
+// ModelForwardSeq(model, device, ids, /*full_output=*/true) (kernels/kernels.h:279-284):
+// logits of every position, [n][vocab] row-major.  Returns the number of floats written.
+long long fr_model_run_full(void *m, const int *ids, int n, float *logits, long long capacity) {
+  return guarded([&]() -> long long {
+    auto *model = static_cast<rwkv::Model *>(m);
+    rwkv::Tensor out = rwkv::Copy(
+        rwkv::ModelForwardSeq(model, model->_act_device, std::vector<int>(ids, ids + n), true), rwkv::Device::kCPU);
+    const long long v = static_cast<long long>(out.numel());
     if (v > capacity) throw FRException("logits buffer too small");
     std::memcpy(logits, out.data_ptr<float>(), sizeof(float) * static_cast<size_t>(v));
     return v;

@@ -113,6 +113,7 @@ Tensor vec_to_device(const std::vector<float> &v, const Shape &shape, DType dtyp
 void build_synthetic(Model *model, const Spec &sp, DType wdtype, ModelExtra &ex) {
   const int C = sp.C, F = sp.F, V = sp.V, L = sp.L;
   const bool v5 = sp.version[0] == '5';
+  const bool v50 = sp.version == "5";  // RWKV-5.0: no gate, one decay / bonus per head
   uint64_t stream_id = 0;
   auto key = [&]() { return splitmix64(sp.seed * 0x100000001B3ull + (++stream_id)); };
   auto push = [&](Tensor t) { model->_params.push_back(std::move(t)); };
@@ -153,8 +154,11 @@ void build_synthetic(Model *model, const Spec &sp, DType wdtype, ModelExtra &ex)
     uniform(C, 0, 1, act, {C}, b + "att.time_mix_k");
     uniform(C, 0, 1, act, {C}, b + "att.time_mix_v");
     uniform(C, 0, 1, act, {C}, b + "att.time_mix_r");
-    if (v5) uniform(C, 0, 1, act, {C}, b + "att.time_mix_g");
-    if (v5) {
+    if (v5 && !v50) uniform(C, 0, 1, act, {C}, b + "att.time_mix_g");
+    if (v50) {
+      uniform(sp.H, -6, 0, DType::kFloat32, {sp.H}, b + "att.time_decay", 2);
+      uniform(sp.H, -1, 1, DType::kFloat32, {sp.H}, b + "att.time_first");
+    } else if (v5) {
       uniform(C, -6, 0, DType::kFloat32, {sp.H, C / sp.H}, b + "att.time_decay", 2);
       uniform(C, -1, 1, DType::kFloat32, {sp.H, C / sp.H}, b + "att.time_first");
     } else {
@@ -164,7 +168,7 @@ void build_synthetic(Model *model, const Spec &sp, DType wdtype, ModelExtra &ex)
     matrix(C, C, b + "att.key.weight");
     matrix(C, C, b + "att.value.weight");
     matrix(C, C, b + "att.receptance.weight");
-    if (v5) matrix(C, C, b + "att.gate.weight");
+    if (v5 && !v50) matrix(C, C, b + "att.gate.weight");
     matrix(C, C, b + "att.output.weight");
     constant(C, 1.f, act, b + "ln2.weight");
     constant(C, 0.f, act, b + "ln2.bias");

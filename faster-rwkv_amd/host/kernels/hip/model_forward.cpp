@@ -33,7 +33,8 @@ struct DecodePlan {
   float *logits_host[2] = {nullptr, nullptr};  // pinned; the graph's last node copies into it
   int32_t *ring = nullptr;                     // pinned; token ids, read by the first kernel
   uint32_t fed = 0;                            // tokens fed so far == the device counter
-  bool v5 = false;                      // RWKV-5.1/5.2: state is (shift, [H,S,S] matrix, shift)
+  bool v5 = false;                      // RWKV-5.x: state is (shift, [H,S,S] matrix, shift)
+  bool v50 = false;                     // RWKV-5.0: no gate, 13 attention parameters
   int H = 0;
   std::vector<Tensor> aa, bb, pp;       // RWKV-4
   std::vector<Tensor> wkv;              // RWKV-5
@@ -56,6 +57,7 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   p->L = model->n_layer();
   p->C = model->n_embd();
   p->v5 = model->version() != "4";
+  p->v50 = model->version() == "5";
   p->H = model->head_size();
   p->F = model->n_ffn() > 0 ? model->n_ffn() : static_cast<int>(model->_params[15].size(1));
   p->V = static_cast<int>(ex.emb_table.size(0));
@@ -128,7 +130,26 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
   FRHIP_CHECK(frhip_embed_ring(ex.emb_table.data_ptr(), p.V, 2 * C, p.ring, DecodePlan::kRing,
                                reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
   size_t pi = 0;
-  for (int l = 0; l < p.L && p.v5; l++) {
+  for (int l = 0; l < p.L && p.v50; l++) {
+    const frhip_weight *kw = find_weight(P[pi + 9]), *vw = find_weight(P[pi + 10]), *rw = find_weight(P[pi + 11]),
+                       *ow = find_weight(P[pi + 12]);
+    RV_CHECK(kw && vw && rw && ow);
+    FRHIP_CHECK(frhip_att_one_v5(C, p.H, p.x.data_ptr(), p.sx_att[cur][l].data_ptr(), p.wkv[l].data_ptr<float>(),
+                                 P[pi].data_ptr(), P[pi + 1].data_ptr(), P[pi + 2].data_ptr<float>(),
+                                 P[pi + 3].data_ptr<float>(), P[pi + 4].data_ptr(), P[pi + 5].data_ptr(),
+                                 P[pi + 6].data_ptr(), P[pi + 7].data_ptr<float>(), P[pi + 8].data_ptr<float>(), kw,
+                                 vw, rw, ow, p.x.data_ptr(), p.sx_att[nxt][l].data_ptr(), p.wkv[l].data_ptr<float>(),
+                                 p.ws.data_ptr(), s));
+    pi += 13;
+    const frhip_weight *fk = find_weight(P[pi + 4]), *fv = find_weight(P[pi + 5]), *frw = find_weight(P[pi + 6]);
+    RV_CHECK(fk && fv && frw);
+    FRHIP_CHECK(frhip_ffn_one(C, F, p.x.data_ptr(), p.sx_ffn[cur][l].data_ptr(), P[pi].data_ptr(),
+                              P[pi + 1].data_ptr(), P[pi + 2].data_ptr(), P[pi + 3].data_ptr(), fk, fv, frw,
+                              p.x.data_ptr(), p.sx_ffn[nxt][l].data_ptr(), (l + 1) % 6 == 0 ? 1 : 0, p.ws.data_ptr(),
+                              s));
+    pi += 7;
+  }
+  for (int l = 0; l < p.L && p.v5 && !p.v50; l++) {
     const frhip_weight *kw = find_weight(P[pi + 10]), *vw = find_weight(P[pi + 11]), *rw = find_weight(P[pi + 12]),
                        *gw = find_weight(P[pi + 13]), *ow = find_weight(P[pi + 14]);
     RV_CHECK(kw && vw && rw && gw && ow);
@@ -177,7 +198,7 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
 Tensor ModelForward(Model *model, Device device, int id) {
   const bool generic = std::getenv("FR_HIP_GENERIC") != nullptr;  // read per call so that one process can compare both paths
   const std::string &ver = model->version();
-  if (generic || !(ver == "4" || ver == "5.1" || ver == "5.2")) return def::ModelForward(model, device, id);
+  if (generic || !(ver == "4" || ver == "5" || ver == "5.1" || ver == "5.2")) return def::ModelForward(model, device, id);
   auto ex = extra_of(model);
   if (!ex->plan) ex->plan = make_plan(model, *ex);
   DecodePlan &p = *ex->plan;
@@ -221,14 +242,14 @@ Tensor ModelForward(Model *model, Device device, int id) {
 
 // Seq mode (reference: kernels/default/model_forward_seq.cpp:48-184): embedding rows are
 // gathered on the device, every layer runs its seq operator over all T rows (MFMA products,
-// chunked WKV scans), and only the last row goes through ln_out and the head.  RWKV-4, which
+// chunked WKV scans), and only the last row goes through ln_out and the head (all rows with
+// full_output).  RWKV-4, which
 // upstream cannot run in seq mode (:111-112), goes through the `att_seq` operator.
 // FR_HIP_SEQ_FALLBACK=1 selects the loop of one-token steps (:34-46) instead.
 Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids, bool full_output) {
   const std::string &ver = model->version();
-  if (std::getenv("FR_HIP_SEQ_FALLBACK") || !(ver == "4" || ver == "5.2"))
+  if (std::getenv("FR_HIP_SEQ_FALLBACK") || !(ver == "4" || ver == "5" || ver == "5.2"))
     return def::ModelForwardSeqFallback(model, device, ids, full_output);
-  RV_CHECK(!full_output) << "full_output is not supported on hip yet";
   RV_CHECK(!ids.empty());
   auto ex = extra_of(model);
   const int T = static_cast<int>(ids.size()), C = model->n_embd();
@@ -252,6 +273,11 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
           att_seq(x, st[0], st[1], st[2], st[3], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5],
                   p[pi + 6], p[pi + 7], p[pi + 8], p[pi + 9], p[pi + 10]);
       pi += 11;
+    } else if (ver == "5") {
+      std::tie(x, st[0], st[1]) =
+          att_seq_v5(x, st[0], st[1], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5], p[pi + 6],
+                     p[pi + 7], p[pi + 8], p[pi + 9], p[pi + 10], p[pi + 11], p[pi + 12]);
+      pi += 13;
     } else {
       std::tie(x, st[0], st[1]) =
           att_seq_v5_2(x, st[0], st[1], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5], p[pi + 6],
@@ -264,9 +290,16 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
     pi += 7;
     if ((i + 1) % 6 == 0) scalar_div_(x, 2);
   }
-  // last row -> ln_out -> head -> fp32 (model_forward_seq.cpp:170-178)
   const frhip_weight *hw = find_weight(p[pi + 2]);
   RV_CHECK(hw != nullptr);
+  if (full_output) {
+    // every row -> ln_out -> head -> fp32 [T, V] (model_forward_seq.cpp:173-178 without the slice)
+    Tensor y = layernorm(x, p[pi], p[pi + 1]);
+    Tensor lg = Tensor::Empty({T, static_cast<LengthType>(hw->N)}, DType::kFloat16, Device::kHIP);
+    FRHIP_CHECK(frhip_gemm(y.data_ptr(), hw, lg.data_ptr(), T, FRHIP_F16, s));
+    return cast_dtype(lg, DType::kFloat32);
+  }
+  // last row -> ln_out -> head -> fp32 (model_forward_seq.cpp:170-178)
   Tensor logits = Tensor::Empty({static_cast<LengthType>(hw->N)}, DType::kFloat32, Device::kHIP);
   const char *last = static_cast<const char *>(x.data_ptr()) + static_cast<size_t>(T - 1) * C * 2;
   FRHIP_CHECK(frhip_head(C, last, p[pi].data_ptr(), p[pi + 1].data_ptr(), hw, logits.data_ptr<float>(), s));

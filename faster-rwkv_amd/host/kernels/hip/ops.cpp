@@ -186,6 +186,33 @@ att_one_v5_1(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &l
   return {x_out, xx, s_out};
 }
 
+// att_one_v5, RWKV-5.0 one token (reference: kernels/cuda/att.cu:362-391).  t_decay and
+// t_first hold one value per head ([H] or [H,1,1]).
+std::tuple<Tensor, Tensor, Tensor>
+att_one_v5(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &ln_w, const Tensor &ln_b,
+           const Tensor &lx_w, const Tensor &lx_b, const Tensor &k_mix, const Tensor &v_mix, const Tensor &r_mix,
+           const Tensor &t_decay, const Tensor &t_first, const Tensor &kw, const Tensor &vw, const Tensor &rw,
+           const Tensor &ow) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 1);
+  const int C = static_cast<int>(x.size(0));
+  const int H = static_cast<int>(t_decay.size(0));
+  RV_CHECK(t_decay.numel() == H && t_first.numel() == H) << "att_one_v5: time_decay/time_first must hold one value per head";
+  frhip_weight d[4];
+  Tensor tmp[4];
+  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
+                              weight_of(ow, d[3], tmp[3])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor s_out = Tensor::Empty(s.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor ws = workspace(C, 16);
+  FRHIP_CHECK(frhip_att_one_v5(C, H, x.data_ptr(), sx.data_ptr(), s.data_ptr<float>(), ln_w.data_ptr(),
+                               ln_b.data_ptr(), lx_w.data_ptr<float>(), lx_b.data_ptr<float>(), k_mix.data_ptr(),
+                               v_mix.data_ptr(), r_mix.data_ptr(), t_decay.data_ptr<float>(),
+                               t_first.data_ptr<float>(), w[0], w[1], w[2], w[3], x_out.data_ptr(), xx.data_ptr(),
+                               s_out.data_ptr<float>(), ws.data_ptr(), stream()));
+  return {x_out, xx, s_out};
+}
+
 static Tensor seq_workspace(int T, int C, int F) {
   return Tensor::Empty({static_cast<LengthType>(frhip_seq_workspace_bytes(T, C, F))}, DType::kInt8, Device::kHIP);
 }
@@ -260,6 +287,32 @@ att_seq_v5_2(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &l
   return {x_out, xx, s_out};
 }
 
+// att_seq_v5, RWKV-5.0 (reference: kernels/cuda/att_seq.cu:425-462).
+std::tuple<Tensor, Tensor, Tensor>
+att_seq_v5(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &ln_w, const Tensor &ln_b,
+           const Tensor &lx_w, const Tensor &lx_b, const Tensor &k_mix, const Tensor &v_mix, const Tensor &r_mix,
+           const Tensor &t_decay, const Tensor &t_first, const Tensor &kw, const Tensor &vw, const Tensor &rw,
+           const Tensor &ow) {
+  RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 2);
+  const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1));
+  const int H = static_cast<int>(t_decay.size(0));
+  RV_CHECK(t_decay.numel() == H && t_first.numel() == H) << "att_seq_v5: time_decay/time_first must hold one value per head";
+  frhip_weight d[4];
+  Tensor tmp[4];
+  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
+                              weight_of(ow, d[3], tmp[3])};
+  Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
+  Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
+  Tensor s_out = Tensor::Empty(s.sizes(), DType::kFloat32, Device::kHIP);
+  Tensor ws = seq_workspace(T, C, 64);
+  FRHIP_CHECK(frhip_att_seq_v5(T, C, H, x.data_ptr(), sx.data_ptr(), s.data_ptr<float>(), ln_w.data_ptr(),
+                               ln_b.data_ptr(), lx_w.data_ptr<float>(), lx_b.data_ptr<float>(), k_mix.data_ptr(),
+                               v_mix.data_ptr(), r_mix.data_ptr(), t_decay.data_ptr<float>(),
+                               t_first.data_ptr<float>(), w[0], w[1], w[2], w[3], x_out.data_ptr(), xx.data_ptr(),
+                               s_out.data_ptr<float>(), ws.data_ptr(), stream()));
+  return {x_out, xx, s_out};
+}
+
 KernelRegister fill_reg("fill_", Device::kHIP, fill_);
 KernelRegister cast_reg("cast_dtype", Device::kHIP, cast_dtype);
 KernelRegister scalar_div_reg("scalar_div_", Device::kHIP, scalar_div_);
@@ -273,6 +326,8 @@ KernelRegister ffn_seq_reg("ffn_seq", Device::kHIP, ffn_seq);
 KernelRegister att_seq_reg("att_seq", Device::kHIP, att_seq);
 KernelRegister att_seq_v5_2_reg("att_seq_v5_2", Device::kHIP, att_seq_v5_2);
 KernelRegister att_one_v5_1_reg("att_one_v5_1", Device::kHIP, att_one_v5_1);
+KernelRegister att_one_v5_reg("att_one_v5", Device::kHIP, att_one_v5);
+KernelRegister att_seq_v5_reg("att_seq_v5", Device::kHIP, att_seq_v5);
 
 }  // namespace hip
 }  // namespace rwkv

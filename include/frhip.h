@@ -159,6 +159,17 @@ int frhip_att_one_v5_1(int C, int H, const void *x, const void *sx, const float 
                        const frhip_weight *gw, const frhip_weight *ow,
                        void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
 
+/* att_one_v5 (RWKV-5.0, one token): kernels/cuda/att.cu:219-265,362-391.  As
+ * frhip_att_one_v5_1 without the gate; t_decay, t_first [H], one value per head
+ * (att.cu:70,73 index them by i / (S*S)). */
+int frhip_att_one_v5(int C, int H, const void *x, const void *sx, const float *s,
+                     const void *ln_w, const void *ln_b, const float *lx_w, const float *lx_b,
+                     const void *k_mix, const void *v_mix, const void *r_mix,
+                     const float *t_decay, const float *t_first,
+                     const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                     const frhip_weight *ow,
+                     void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
+
 /* ---- seq-mode (prompt) operators ---------------------------------------------- */
 /* matmul, matrix x matrix: kernels/cuda/matmul.cpp:110-121.  x [T][K] binary16, y [T][N] in
  * out_dtype (F16 or F32); fp32 accumulation on the MFMA units.  K must be a multiple of 64. */
@@ -197,6 +208,15 @@ int frhip_att_seq_v5_2(int T, int C, int H, const void *x, const void *sx, const
                        const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
                        const frhip_weight *gw, const frhip_weight *ow,
                        void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
+
+/* att_seq_v5 (RWKV-5.0): kernels/cuda/att_seq.cu:158-256,425-462.  t_decay, t_first [H]. */
+int frhip_att_seq_v5(int T, int C, int H, const void *x, const void *sx, const float *s,
+                     const void *ln_w, const void *ln_b, const float *lx_w, const float *lx_b,
+                     const void *k_mix, const void *v_mix, const void *r_mix,
+                     const float *t_decay, const float *t_first,
+                     const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                     const frhip_weight *ow,
+                     void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
 
 /* ---- bandwidth probes (measurement aids, no counterpart in the reference) --------- */
 /* Plain device copy, 16 bytes per lane: the kernel of known traffic (bytes read + bytes

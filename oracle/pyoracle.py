@@ -78,6 +78,9 @@ _sig("orc_ffn_seq_f16", None, *([_vp] * 11), _i, _i, _i)
 _sig("orc_att_one_v5_1_f16", None, *([_vp] * 20), _i, _i)
 _sig("orc_att_seq_v5_2_f16", None, *([_vp] * 20), _i, _i, _i)
 _sig("orc_wkv5_2_seq_f32", None, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i)
+_sig("orc_att_one_v5_f16", None, *([_vp] * 18), _i, _i)
+_sig("orc_att_seq_v5_f16", None, *([_vp] * 18), _i, _i, _i)
+_sig("orc_wkv5_seq_matrix_f32", None, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i)
 _sig("orc_argmax", _i, _vp, _i)
 
 
@@ -232,6 +235,31 @@ def att_v5_2_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, mg, td, tf, kw, v
     else:
         lib.orc_att_seq_v5_2_f16(*args, x.shape[0], C_, H)
     return x_out, xx, s
+
+
+def att_v5_0_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, td, tf, kw, vw, rw, ow, H):
+    """RWKV-5.0.  One token (x.ndim==1: att.cu:362-391) or sequence in matrix form
+    (att_seq.cu:425-462) -> (x_out, xx_last, s')."""
+    C_ = x.shape[-1]
+    s = s.copy()
+    x_out = np.empty_like(x)
+    xx = np.empty(C_, np.float16)
+    args = [_p(a) for a in (x, sx, s, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, td, tf, kw, vw, rw, ow, x_out, xx)]
+    if x.ndim == 1:
+        lib.orc_att_one_v5_f16(*args, C_, H)
+    else:
+        lib.orc_att_seq_v5_f16(*args, x.shape[0], C_, H)
+    return x_out, xx, s
+
+
+def wkv5_seq_matrix_f32(s, r, k, v, w, u):
+    """att_seq.cu:181-243 (RWKV-5.0 matrix form); w, u [H]."""
+    T, C_ = r.shape
+    H = w.shape[0]
+    s = s.copy()
+    y = np.empty((T, C_), np.float32)
+    lib.orc_wkv5_seq_matrix_f32(_p(s), _p(r), _p(k), _p(v), _p(w), _p(u), _p(y), T, H, C_ // H)
+    return y, s
 
 
 def wkv5_2_seq_f32(s, r, k, v, w, u):

@@ -9,6 +9,7 @@
 #include "rwkv_oracle.h"
 
 #include <math.h>
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -485,7 +486,8 @@ static void att_v5_2_tail_f16(const orc_half *x, const float *wkv_out, const flo
   orc_half *gh = (orc_half *)xmalloc(2 * n), *out = (orc_half *)xmalloc(2 * n);
   orc_groupnorm_f32(wkv_out, H, lx_w, lx_b, gn, T, C);
   orc_f2h_n(gn, gh, n);
-  for (size_t i = 0; i < n; i++) gh[i] = orc_hmul(gh[i], g[i]);
+  if (g) /* RWKV-5.0 has no gate: att.cu:258-259 */
+    for (size_t i = 0; i < n; i++) gh[i] = orc_hmul(gh[i], g[i]);
   orc_gemm_f16(gh, ow, NULL, out, T, C, C);
   for (size_t i = 0; i < n; i++) x_out[i] = orc_hadd(x[i], out[i]);
   free(gn); free(gh); free(out);
@@ -548,6 +550,111 @@ void orc_att_seq_v5_2_f16(const orc_half *x, const orc_half *sx, float *s, const
                           orc_half *xx_last_out, int T, int C, int H) {
   att_v5_2_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, g_mix, t_decay, t_first, kw,
                vw, rw, gw, ow, x_out, xx_last_out, T, C, H, 1);
+}
+
+/* RWKV-5.0 sequence recurrence in the reference's matrix form (att_seq.cu:181-243), per head
+ * with scalar decay w and bonus u:
+ *   out_t = sum_{i<t} (r_t.k_i) w^(t-1-i) v_i + u (r_t.k_t) v_t + (r_t S) w^t
+ *   S'    = w^T S + sum_i w^(T-1-i) k_i v_i^T
+ * powers through powf as the reference's __powf functors (att_seq.cu:142-155). */
+void orc_wkv5_seq_matrix_f32(float *s, const float *r, const float *k, const float *v,
+                             const float *w, const float *u, float *y, int T, int H, int S) {
+  int C = H * S;
+  float *rk = (float *)xmalloc(4 * (size_t)T * T), *rs = (float *)xmalloc(4 * (size_t)T * S);
+  float *sn = (float *)xmalloc(4 * (size_t)S * S);
+  for (int h = 0; h < H; h++) {
+    float *sh = s + (size_t)h * S * S;
+    const float wh = w[h], uh = u[h];
+    for (int t = 0; t < T; t++) {
+      const float *rt = r + (size_t)t * C + h * S;
+      for (int i = 0; i <= t; i++) {
+        const float *ki = k + (size_t)i * C + h * S;
+        float acc = 0.f;
+        for (int c = 0; c < S; c++) acc += rt[c] * ki[c];
+        float wt = i == t ? uh : powf(wh, (float)(t - 1 - i)); /* att_seq.cu:193-201 */
+        rk[(size_t)t * T + i] = acc * wt;
+      }
+      for (int j = 0; j < S; j++) {
+        float acc = 0.f;
+        for (int c = 0; c < S; c++) acc += rt[c] * sh[c * S + j];
+        rs[(size_t)t * S + j] = acc * powf(wh, (float)t); /* wb: att_seq.cu:192,222-225 */
+      }
+    }
+    for (int t = 0; t < T; t++)
+      for (int j = 0; j < S; j++) {
+        float acc = 0.f;
+        for (int i = 0; i <= t; i++) acc += rk[(size_t)t * T + i] * v[(size_t)i * C + h * S + j];
+        y[(size_t)t * C + h * S + j] = acc + rs[(size_t)t * S + j]; /* att_seq.cu:227-231 */
+      }
+    const float wT = powf(wh, (float)T); /* att_seq.cu:183-186 */
+    for (int c = 0; c < S; c++)
+      for (int j = 0; j < S; j++) {
+        float acc = 0.f;
+        for (int i = 0; i < T; i++)
+          acc += (k[(size_t)i * C + h * S + c] * powf(wh, (float)(T - 1 - i))) * v[(size_t)i * C + h * S + j];
+        sn[c * S + j] = wT * sh[c * S + j] + acc; /* att_seq.cu:232-243 */
+      }
+    memcpy(sh, sn, 4 * (size_t)S * S);
+  }
+  free(rk); free(rs); free(sn);
+}
+
+/* RWKV-5.0 attention: one token kernels/cuda/att.cu:219-265,362-391 (matrix_form 0),
+ * sequence kernels/cuda/att_seq.cu:158-256,425-462 (matrix_form 1).  t_decay, t_first [H]. */
+static void att_v5_0_f16(const orc_half *x, const orc_half *sx, float *s, const orc_half *ln_w,
+                         const orc_half *ln_b, const float *lx_w, const float *lx_b,
+                         const orc_half *k_mix, const orc_half *v_mix, const orc_half *r_mix,
+                         const float *t_decay, const float *t_first, const orc_half *kw,
+                         const orc_half *vw, const orc_half *rw, const orc_half *ow,
+                         orc_half *x_out, orc_half *xx_last_out, int T, int C, int H,
+                         int matrix_form) {
+  size_t n = (size_t)T * C;
+  int S = C / H;
+  orc_half *xx = (orc_half *)xmalloc(2 * n), *sh = (orc_half *)xmalloc(2 * n);
+  orc_half *kx = (orc_half *)xmalloc(2 * n), *vx = (orc_half *)xmalloc(2 * n), *rx = (orc_half *)xmalloc(2 * n);
+  float *k = (float *)xmalloc(4 * n), *v = (float *)xmalloc(4 * n), *r = (float *)xmalloc(4 * n);
+  float *y = (float *)xmalloc(4 * n);
+  orc_layernorm_f16(x, ln_w, ln_b, xx, T, C);
+  shift_rows_f16(sx, xx, sh, T, C);
+  orc_mix_f16(xx, sh, k_mix, kx, T, C);
+  orc_mix_f16(xx, sh, v_mix, vx, T, C);
+  orc_mix_f16(xx, sh, r_mix, rx, T, C);
+  orc_gemm_f16(kx, kw, k, NULL, T, C, C);
+  orc_gemm_f16(vx, vw, v, NULL, T, C, C);
+  orc_gemm_f16(rx, rw, r, NULL, T, C, C);
+  if (matrix_form) {
+    orc_wkv5_seq_matrix_f32(s, r, k, v, t_decay, t_first, y, T, H, S);
+  } else {
+    /* OneV5MulAdd indexes t_first, t_decay by i / (S*S) (att.cu:70,73): one value per head */
+    float *wx = (float *)xmalloc(4 * (size_t)C), *ux = (float *)xmalloc(4 * (size_t)C);
+    for (int i = 0; i < C; i++) { wx[i] = t_decay[i / S]; ux[i] = t_first[i / S]; }
+    for (int t = 0; t < T; t++)
+      wkv5_one_f32(s, r + (size_t)t * C, k + (size_t)t * C, v + (size_t)t * C, wx, ux, y + (size_t)t * C, H, S);
+    free(wx); free(ux);
+  }
+  att_v5_2_tail_f16(x, y, lx_w, lx_b, NULL, ow, x_out, T, C, H);
+  memcpy(xx_last_out, xx + (size_t)(T - 1) * C, sizeof(orc_half) * (size_t)C);
+  free(xx); free(sh); free(kx); free(vx); free(rx); free(k); free(v); free(r); free(y);
+}
+
+void orc_att_one_v5_f16(const orc_half *x, const orc_half *sx, float *s, const orc_half *ln_w,
+                        const orc_half *ln_b, const float *lx_w, const float *lx_b,
+                        const orc_half *k_mix, const orc_half *v_mix, const orc_half *r_mix,
+                        const float *t_decay, const float *t_first, const orc_half *kw,
+                        const orc_half *vw, const orc_half *rw, const orc_half *ow,
+                        orc_half *x_out, orc_half *xx_out, int C, int H) {
+  att_v5_0_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, t_decay, t_first, kw, vw, rw,
+               ow, x_out, xx_out, 1, C, H, 0);
+}
+
+void orc_att_seq_v5_f16(const orc_half *x, const orc_half *sx, float *s, const orc_half *ln_w,
+                        const orc_half *ln_b, const float *lx_w, const float *lx_b,
+                        const orc_half *k_mix, const orc_half *v_mix, const orc_half *r_mix,
+                        const float *t_decay, const float *t_first, const orc_half *kw,
+                        const orc_half *vw, const orc_half *rw, const orc_half *ow,
+                        orc_half *x_out, orc_half *xx_last_out, int T, int C, int H) {
+  att_v5_0_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, k_mix, v_mix, r_mix, t_decay, t_first, kw, vw, rw,
+               ow, x_out, xx_last_out, T, C, H, 1);
 }
 
 /* ======================================================================== */
@@ -696,6 +803,20 @@ static void forward_seq_f16(const orc_model *m, void *const *state, const int *i
                       (const orc_half *)p[5], (const orc_half *)p[6], x, xx_last, T, C, F);
       memcpy(st[4], xx_last, 2 * (size_t)C);
       p += 7;
+    } else if (m->version == 50) { /* model_forward.cpp:124-137, model_forward_seq.cpp:113-126 */
+      att_v5_0_f16(x, (const orc_half *)st[0], (float *)st[1], (const orc_half *)p[0],
+                   (const orc_half *)p[1], (const float *)p[2], (const float *)p[3],
+                   (const orc_half *)p[4], (const orc_half *)p[5], (const orc_half *)p[6],
+                   (const float *)p[7], (const float *)p[8], (const orc_half *)p[9],
+                   (const orc_half *)p[10], (const orc_half *)p[11], (const orc_half *)p[12], y,
+                   xx_last, T, C, m->n_head, T > 1);
+      memcpy(st[0], xx_last, 2 * (size_t)C);
+      p += 13;
+      orc_ffn_seq_f16(y, (const orc_half *)st[2], (const orc_half *)p[0], (const orc_half *)p[1],
+                      (const orc_half *)p[2], (const orc_half *)p[3], (const orc_half *)p[4],
+                      (const orc_half *)p[5], (const orc_half *)p[6], x, xx_last, T, C, F);
+      memcpy(st[2], xx_last, 2 * (size_t)C);
+      p += 7;
     } else {
       att_v5_2_f16(x, (const orc_half *)st[0], (float *)st[1], (const orc_half *)p[0],
                    (const orc_half *)p[1], (const float *)p[2], (const float *)p[3],
@@ -735,6 +856,9 @@ static void forward_one_f32(const orc_model *m, void *const *state, int id, floa
       p += 11;
       ffn_one_f32(y, (float *)st[4], p, x, C, F);
       p += 7;
+    } else if (m->version == 50) {
+      fprintf(stderr, "rwkv_oracle: RWKV-5.0 is restated in ORC_F16 mode only\n");
+      abort();
     } else {
       att_one_v5_2_f32(x, (float *)st[0], (float *)st[1], p, y, C, m->n_head);
       p += 15;

@@ -116,7 +116,27 @@ void orc_att_one_v5_1_f16(const orc_half *x, const orc_half *sx, float *s, const
                           const orc_half *gw, const orc_half *ow, orc_half *x_out,
                           orc_half *xx_out, int C, int H);
 
+/* kernels/cuda/att.cu:219-265,362-391 (RWKV-5.0: no gate; t_decay, t_first [H], one value
+ * per head). */
+void orc_att_one_v5_f16(const orc_half *x, const orc_half *sx, float *s, const orc_half *ln_w,
+                        const orc_half *ln_b, const float *lx_w, const float *lx_b,
+                        const orc_half *k_mix, const orc_half *v_mix, const orc_half *r_mix,
+                        const float *t_decay, const float *t_first, const orc_half *kw,
+                        const orc_half *vw, const orc_half *rw, const orc_half *ow,
+                        orc_half *x_out, orc_half *xx_out, int C, int H);
+
 /* ---- layer-level ops (sequence of T tokens) ------------------------------ */
+/* kernels/cuda/att_seq.cu:181-243: the RWKV-5.0 recurrence over T tokens in matrix form.
+ * w, u [H]; s [H][S key][S value] updated in place; y [T][H*S]. */
+void orc_wkv5_seq_matrix_f32(float *s, const float *r, const float *k, const float *v,
+                             const float *w, const float *u, float *y, int T, int H, int S);
+/* kernels/cuda/att_seq.cu:158-256,425-462. */
+void orc_att_seq_v5_f16(const orc_half *x, const orc_half *sx, float *s, const orc_half *ln_w,
+                        const orc_half *ln_b, const float *lx_w, const float *lx_b,
+                        const orc_half *k_mix, const orc_half *v_mix, const orc_half *r_mix,
+                        const float *t_decay, const float *t_first, const orc_half *kw,
+                        const orc_half *vw, const orc_half *rw, const orc_half *ow,
+                        orc_half *x_out, orc_half *xx_last_out, int T, int C, int H);
 /* kernels/cuda/ffn_seq.cu:65-109.  x [T,C]; sx [C] is the shift state; xx_last_out
  * receives LN(x)[T-1] (the new shift state). */
 void orc_ffn_seq_f16(const orc_half *x, const orc_half *sx, const orc_half *ln_w,
@@ -147,13 +167,15 @@ void orc_att_seq_v4_f16(const orc_half *x, const orc_half *sx, float *aa, float 
 
 /* ---- whole model ---------------------------------------------------------- */
 typedef struct {
-  int version; /* 4 or 52 (RWKV-5.2) */
+  int version; /* 4, 50 (RWKV-5.0, ORC_F16 only) or 52 (RWKV-5.1/5.2) */
   int mode;    /* ORC_F32 or ORC_F16 */
   int n_layer, n_embd, n_att, n_ffn, n_head, vocab;
   /* Parameters in the reference's positional order
    * (kernels/default/init_model.cpp:91-126): per layer
    *   v4 : ln1.w ln1.b  tmk tmv tmr  time_decay time_first  Wk Wv Wr Wo
    *        ln2.w ln2.b  ffn.tmk ffn.tmr  ffn.Wk ffn.Wv ffn.Wr                (18)
+   *   5.0: ln1.w ln1.b ln_x.w ln_x.b tmk tmv tmr time_decay time_first
+   *        Wk Wv Wr Wo  ln2.w ln2.b ffn.tmk ffn.tmr ffn.Wk ffn.Wv ffn.Wr       (20)
    *   5.2: ln1.w ln1.b ln_x.w ln_x.b tmk tmv tmr tmg time_decay time_first
    *        Wk Wv Wr Wg Wo  ln2.w ln2.b ffn.tmk ffn.tmr ffn.Wk ffn.Wv ffn.Wr   (22)
    * then ln_out.w ln_out.b head.weight.

@@ -4,7 +4,8 @@ configurations: 2-D weights ~N(0, 0.02); time_decay_raw ~U(-5,1) (v4) / U(-6,0)
 (v5.2); time_first ~U(-1,1); time_mix ~U(0,1); layernorm gamma=1, beta=0 (tests
 perturb gamma/beta slightly so that the affine part is exercised).
 Stored forms are the ones the kernels consume: v4 time_decay = -exp(raw) (fp32);
-v5.2 time_decay = exp(-exp(raw)) [H,S] (fp32); matrices [in,out].
+v5.2 time_decay = exp(-exp(raw)) [H,S] (fp32), v5.0 (version=50) the same with one
+value per head [H] and no gate; matrices [in,out].
 """
 import numpy as np
 
@@ -38,6 +39,13 @@ def make_model(version, L, C, F, V, H=0, seed=0, dtype=np.float16, affine_jitter
             params += [mixv(), mixv(), mixv()]
             params += [(-np.exp(rng.uniform(-5, 1, C))).astype(np.float32),
                        rng.uniform(-1, 1, C).astype(np.float32)]
+            params += [mat(C, C), mat(C, C), mat(C, C), mat(C, C)]
+        elif version == 50:
+            params += [(1.0 + affine_jitter * rng.standard_normal(C)).astype(np.float32),
+                       (affine_jitter * rng.standard_normal(C)).astype(np.float32)]
+            params += [mixv(), mixv(), mixv()]
+            params += [np.exp(-np.exp(rng.uniform(-6, 0, H))).astype(np.float32),
+                       rng.uniform(-1, 1, H).astype(np.float32)]
             params += [mat(C, C), mat(C, C), mat(C, C), mat(C, C)]
         else:
             S = C // H
@@ -78,12 +86,13 @@ def quantize_u8(w):
 
 
 MATRIX_POS_V4 = (7, 8, 9, 10, 15, 16, 17)
+MATRIX_POS_V50 = (9, 10, 11, 12, 17, 18, 19)
 MATRIX_POS_V52 = (10, 11, 12, 13, 14, 19, 20, 21)
 
 
 def matrix_indices(version, L):
-    per = 18 if version == 4 else 22
-    pos = MATRIX_POS_V4 if version == 4 else MATRIX_POS_V52
+    per = {4: 18, 50: 20}.get(version, 22)
+    pos = {4: MATRIX_POS_V4, 50: MATRIX_POS_V50}.get(version, MATRIX_POS_V52)
     idx = [l * per + p for l in range(L) for p in pos]
     idx.append(L * per + 2)  # head.weight
     return idx

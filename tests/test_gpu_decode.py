@@ -140,6 +140,37 @@ def test_att_one_v5_1(C_, H_, quant):
     assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
 
 
+@pytest.mark.parametrize("C_,H_", [(2048, 32), (512, 8)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_att_one_v5(C_, H_, quant):
+    """RWKV-5.0, kernels/cuda/att.cu:219-265,362-391: no gate, one decay / bonus per head."""
+    S_ = C_ // H_
+    x, sx = h(rng.standard_normal(C_) * 2), h(rng.standard_normal(C_))
+    s = rng.standard_normal((H_, S_, S_)).astype(np.float32)
+    ln_w, ln_b = h(1 + 0.1 * rng.standard_normal(C_)), h(0.1 * rng.standard_normal(C_))
+    lx_w = (1 + 0.1 * rng.standard_normal(C_)).astype(np.float32)
+    lx_b = (0.1 * rng.standard_normal(C_)).astype(np.float32)
+    mixes = [h(rng.uniform(0, 1, C_)) for _ in range(3)]
+    td = np.exp(-np.exp(rng.uniform(-6, 0, H_))).astype(np.float32)
+    tf = rng.uniform(-1, 1, H_).astype(np.float32)
+    ws, refs = [], []
+    for _ in range(4):
+        w, r = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+        ws.append(w)
+        refs.append(r)
+    ref_x, ref_xx, ref_s = po.att_v5_0_f16(x, sx, s, ln_w, ln_b, lx_w, lx_b, *mixes, td, tf, *refs, H_)
+    x_out, xx_out = DevBuf.empty(C_, np.float16), DevBuf.empty(C_, np.float16)
+    s_out = DevBuf.empty((H_, S_, S_), np.float32)
+    wsb = DevBuf(L().frhip_decode_workspace_bytes(C_, 4 * C_))
+    fr.check(L().frhip_att_one_v5(C_, H_, keep(x).ptr, keep(sx).ptr, keep(s).ptr, keep(ln_w).ptr, keep(ln_b).ptr,
+                                  keep(lx_w).ptr, keep(lx_b).ptr, *[keep(m).ptr for m in mixes], keep(td).ptr,
+                                  keep(tf).ptr, *[w.ref for w in ws], x_out.ptr, xx_out.ptr, s_out.ptr, wsb.ptr,
+                                  None))
+    assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx")
+    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-5, atol=1e-5)
+    assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
+
+
 @pytest.mark.parametrize("quant", [False, True])
 def test_head(quant):
     C_, V_ = 2048, 65536

@@ -171,3 +171,63 @@ def test_rwkv5_2_model_matches_oracle(tmp_path):
             assert np.abs(ls - lo).max() <= 2e-2
             tok = int(np.argmax(lo))
         m.close()
+
+
+def test_rwkv5_0_model_matches_oracle(tmp_path):
+    """RWKV-5.0 through Model::Run: fused one-token path, seq mode, and the operator loop."""
+    L5, C5, F5, V5, H5 = 6, 512, 1792, 2048, 8
+    params, emb = make_model(50, L5, C5, F5, V5, H5, seed=23)
+    path = str(tmp_path / "v50.fr")
+    fr.write_fr(path, "5", L5, C5, F5, H5, params, emb)
+    for strategy in ("hip fp16", "hip int8"):
+        p = list(params)
+        if strategy.endswith("int8"):
+            for i in matrix_indices(50, L5):
+                p[i] = po.dequant_u8(*quantize_u8(params[i]))
+        om = po.Model(50, po.F16, L5, C5, F5, H5, V5, p, emb)
+        m = fr.Model(path, strategy)
+        assert m.n_head == H5 and m.n_ffn == F5
+        tok, worst = 11, 0.0
+        for step in range(48):
+            lh, lo = m.run(tok), om.run(tok)
+            worst = max(worst, float(np.abs(lh - lo).max()))
+            if int(np.argmax(lh)) != int(np.argmax(lo)):
+                # only a tie at the resolution of binary16 logits (one spacing near 1.0 is 9.8e-4) may differ
+                margin = float(lo.max() - lo[int(np.argmax(lh))])
+                assert margin <= 1e-3, "greedy token differs at step %d (oracle margin %g)" % (step, margin)
+            tok = int(np.argmax(lo))
+        print(strategy, "v5.0 worst |dlogit| over 48 steps:", worst, flush=True)
+        assert worst <= 2e-2
+        s_ref = om.state[5 * 3 + 1]
+        s_got = m.state(5, 1, np.float32)
+        assert np.abs(s_got - s_ref).max() <= 5e-3 * np.abs(s_ref).max()
+        m.reset()
+        om.reset()
+        prompt = [int(t) for t in np.random.default_rng(45).integers(0, V5, 80)]
+        ls, lo = m.run(prompt), om.run(prompt)
+        assert np.abs(ls - lo).max() <= 2e-2 and int(np.argmax(ls)) == int(np.argmax(lo))
+        tok = int(np.argmax(lo))
+        for step in range(8):
+            ls, lo = m.run(tok), om.run(tok)
+            assert np.abs(ls - lo).max() <= 2e-2
+            tok = int(np.argmax(lo))
+        m.close()
+
+
+def test_full_output_gives_the_logits_of_every_position(model_files):
+    """ModelForwardSeq(..., full_output=true) (kernels/default/model_forward_seq.cpp:170-178): row t
+    equals the logits of a run over the first t+1 tokens; the last row equals Model::Run."""
+    path, params, emb = model_files
+    m = fr.Model(path, "hip fp16")
+    om = po.Model(4, po.F16, L_, C_, F_, 0, V_, params, emb)
+    prompt = [int(t) for t in np.random.default_rng(46).integers(0, V_, 40)]
+    full = m.run_full(prompt)
+    assert full.shape == (40, V_)
+    m.reset()
+    last = m.run(prompt)
+    assert np.abs(full[-1] - last).max() <= 1e-3
+    for t in (0, 7, 39):
+        om.reset()
+        lo = om.run(prompt[: t + 1]) if t else om.run(prompt[0])
+        assert np.abs(full[t] - lo).max() <= 2e-2 and int(np.argmax(full[t])) == int(np.argmax(lo))
+    m.close()

@@ -156,3 +156,36 @@ def test_att_seq_v5_2(T, C_, H_, quant):
     assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx_last")
     assert np.allclose(s_out.numpy(), ref_s, rtol=1e-4, atol=1e-4 * np.abs(ref_s).max())
     assert_close_f16(x_out.numpy().reshape(ref_x.shape), ref_x, max_ulp=4, max_frac=0.2, what="x_out", floor_rms=1.0)
+
+
+@pytest.mark.parametrize("T,C_,H_", [(48, 512, 8), (300, 2048, 32), (1, 512, 8), (77, 512, 8)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_att_seq_v5(T, C_, H_, quant):
+    """RWKV-5.0 seq attention against the oracle's matrix form (kernels/cuda/att_seq.cu:158-256)."""
+    if C_ == 2048 and quant:
+        pytest.skip("full-size case runs once")
+    S_ = C_ // H_
+    x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
+    s = rng.standard_normal((H_, S_, S_)).astype(np.float32)
+    ln_w, ln_b = _common(C_)
+    lx_w = (1 + 0.1 * rng.standard_normal(C_)).astype(np.float32)
+    lx_b = (0.1 * rng.standard_normal(C_)).astype(np.float32)
+    mixes = [h(rng.uniform(0, 1, C_)) for _ in range(3)]
+    td = np.exp(-np.exp(rng.uniform(-6, 0, H_))).astype(np.float32)
+    tf = rng.uniform(-1, 1, H_).astype(np.float32)
+    ws_, refs = [], []
+    for _ in range(4):
+        w, r = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+        ws_.append(w)
+        refs.append(r)
+    ref_x, ref_xx, ref_s = po.att_v5_0_f16(x if T > 1 else x[0], sx, s, ln_w, ln_b, lx_w, lx_b, *mixes, td, tf, *refs, H_)
+    x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
+    s_out = DevBuf.empty((H_, S_, S_), np.float32)
+    ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, 4 * C_))
+    fr.check(L().frhip_att_seq_v5(T, C_, H_, keep(x).ptr, keep(sx).ptr, keep(s).ptr, keep(ln_w).ptr, keep(ln_b).ptr,
+                                  keep(lx_w).ptr, keep(lx_b).ptr, *[keep(m).ptr for m in mixes], keep(td).ptr,
+                                  keep(tf).ptr, *[w.ref for w in ws_], x_out.ptr, xx_out.ptr, s_out.ptr, ws.ptr,
+                                  None))
+    assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx_last")
+    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-4, atol=1e-4 * np.abs(ref_s).max())
+    assert_close_f16(x_out.numpy().reshape(ref_x.shape), ref_x, max_ulp=4, max_frac=0.2, what="x_out", floor_rms=1.0)

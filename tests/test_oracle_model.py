@@ -15,7 +15,7 @@ def _model(version, mode, L=3, C=128, F=512, V=300, H=2, seed=3):
     return po.Model(version, mode, L, C, F, H, V, params, emb), params, emb
 
 
-@pytest.mark.parametrize("version", [4, 52])
+@pytest.mark.parametrize("version", [4, 50, 52])
 def test_seq_equals_loop_of_one(version):
     m, _, _ = _model(version, po.F16)
     ids = [5, 17, 299, 0, 42, 7, 7, 123]
@@ -33,7 +33,7 @@ def test_seq_equals_loop_of_one(version):
             assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("version", [4, 52])
+@pytest.mark.parametrize("version", [4, 50, 52])
 def test_reset_then_rerun_is_bit_identical(version):
     m, _, _ = _model(version, po.F16)
     a = [m.run(i).copy() for i in (1, 2, 3)]

@@ -217,6 +217,61 @@ def test_wkv5_scan_matches_brute_force_and_explicit_sum():
         assert np.allclose(s[hd], ex, rtol=1e-4, atol=1e-4)
 
 
+def test_wkv5_0_matrix_form_matches_brute_force_scan():
+    """RWKV-5.0 (att_seq.cu:181-243): the matrix form with decay powers must equal the
+    recurrence with one decay / bonus per head, outputs and final state."""
+    T, H, S = 11, 3, 64
+    C = H * S
+    r, k, v = (rng.standard_normal((T, C)).astype(np.float32) for _ in range(3))
+    w = np.exp(-np.exp(rng.uniform(-6, 0, H))).astype(np.float32)
+    u = rng.uniform(-1, 1, H).astype(np.float32)
+    s0 = rng.standard_normal((H, S, S)).astype(np.float32)
+    y, s = po.wkv5_seq_matrix_f32(s0, r, k, v, w, u)
+    wb = np.repeat(w[:, None], S, axis=1).astype(np.float64)
+    ub = np.repeat(u[:, None], S, axis=1).astype(np.float64)
+    yb, sb = _wkv5_brute(*(a.astype(np.float64) for a in (r, k, v)), wb, ub, s0)
+    assert np.allclose(y, yb, rtol=2e-4, atol=2e-4)
+    assert np.allclose(s, sb, rtol=2e-4, atol=2e-4)
+    # T = 1: out = r.(u k v^T + S), S' = w S + k v^T exactly as the one-token functor (att.cu:64-81)
+    y1, s1 = po.wkv5_seq_matrix_f32(s0, r[:1], k[:1], v[:1], w, u)
+    for hd in range(H):
+        sl = slice(hd * S, (hd + 1) * S)
+        a = np.outer(k[0, sl], v[0, sl]).astype(np.float64)
+        assert np.allclose(y1[0, sl], r[0, sl].astype(np.float64) @ (u[hd] * a + s0[hd]), rtol=1e-4, atol=1e-4)
+        assert np.allclose(s1[hd], w[hd] * s0[hd].astype(np.float64) + a, rtol=1e-5, atol=1e-5)
+
+
+def test_att_v5_0_seq_equals_loop_of_one_token_steps():
+    """The cross-formulation invariant of RWKV-5.0: att_seq_v5 (matrix form) over T rows equals
+    T calls of att_one_v5 (functor form) carrying the state (model_forward_seq.cpp:34-46)."""
+    T, H, S = 7, 2, 64
+    C = H * S
+    h = np.float16
+    x = rng.standard_normal((T, C)).astype(h)
+    sx = rng.standard_normal(C).astype(h)
+    s0 = (0.1 * rng.standard_normal((H, S, S))).astype(np.float32)
+    ln_w, ln_b = (1 + 0.05 * rng.standard_normal(C)).astype(h), (0.05 * rng.standard_normal(C)).astype(h)
+    lx_w, lx_b = (1 + 0.05 * rng.standard_normal(C)).astype(np.float32), (0.05 * rng.standard_normal(C)).astype(np.float32)
+    mk, mv, mr = (rng.uniform(0, 1, C).astype(h) for _ in range(3))
+    td = np.exp(-np.exp(rng.uniform(-6, 0, H))).astype(np.float32)
+    tf = rng.uniform(-1, 1, H).astype(np.float32)
+    kw, vw, rw, ow = ((0.05 * rng.standard_normal((C, C))).astype(h) for _ in range(4))
+    ys, xxs, ss = po.att_v5_0_f16(x, sx, s0, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, td, tf, kw, vw, rw, ow, H)
+    s, shift = s0, sx
+    for t in range(T):
+        y1, shift, s = po.att_v5_0_f16(x[t], shift, s, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, td, tf, kw, vw, rw, ow, H)
+        d = np.abs(y1.astype(np.float32) - ys[t].astype(np.float32)).max()
+        assert d <= 4e-3, (t, d)
+    assert np.array_equal(shift, xxs)
+    assert np.allclose(s, ss, rtol=1e-4, atol=1e-4)
+    # without a gate and with w, u constant over a head, the 5.1 functor path gives the same token
+    y51, _, s51 = po.att_v5_2_f16(x[0], sx, s0, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, mr,
+                                  np.repeat(td[:, None], S, 1), np.repeat(tf[:, None], S, 1), kw, vw, rw,
+                                  np.zeros((C, C), h), ow, H)
+    _, _, s50 = po.att_v5_0_f16(x[0], sx, s0, ln_w, ln_b, lx_w, lx_b, mk, mv, mr, td, tf, kw, vw, rw, ow, H)
+    assert np.array_equal(s51, s50)  # same state update; the outputs differ by the gate
+
+
 # ---------------------------------------------------------------- dequant u8
 def _dequant_numpy(q, mx, rx, my, ry):
     """Independent numpy-float16 statement of the dequantisation: every operation in
