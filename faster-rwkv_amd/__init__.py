@@ -242,6 +242,13 @@ def host():
         h.fr_model_run.argtypes = [_vp, _vp, _i, _vp, _i]
         h.fr_model_run_full.restype = C.c_longlong
         h.fr_model_run_full.argtypes = [_vp, _vp, _i, _vp, C.c_longlong]
+        h.fr_sampler_create.restype = _vp
+        h.fr_sampler_create.argtypes = [_i, _i]
+        h.fr_sampler_free.argtypes = [_vp]
+        h.fr_sampler_set_seed.argtypes = [_vp, _i]
+        h.fr_sampler_sample.argtypes = [_vp, _vp, _i, C.c_float, _i, C.c_float]
+        h.fr_sample_decode.restype = C.c_longlong
+        h.fr_sample_decode.argtypes = [_vp, _vp, _i, _i, C.c_float, _i, C.c_float, _vp]
         h.fr_model_reset.argtypes = [_vp]
         h.fr_model_save_state.argtypes = [_vp, C.c_char_p]
         h.fr_model_load_state.argtypes = [_vp, C.c_char_p]
@@ -301,6 +308,15 @@ class Model:
         n = self._chk(self._h.fr_model_get_state(self._m, layer, index, buf.ctypes.data, buf.size))
         return buf[:n].view(dtype).copy()
 
+    def generate(self, sampler, first_id, steps, temperature=1.0, top_k=0, top_p=1.0):
+        """chat.cpp:56-92 without its penalties, in C++; returns (token ids, seconds)."""
+        out = np.empty(steps, np.int32)
+        us = self._h.fr_sample_decode(self._m, sampler._s, int(first_id), int(steps), temperature, top_k, top_p,
+                                      out.ctypes.data)
+        if us < 0:
+            raise FrhipError(self._h.fr_last_error().decode())
+        return out, us * 1e-6
+
     def greedy(self, first_id, steps):
         """chat.cpp's greedy loop in C++; returns (token ids, seconds)."""
         out = np.empty(steps, np.int32)
@@ -319,6 +335,32 @@ class Model:
             self.close()
         except Exception:
             pass
+
+
+class Sampler:
+    """rwkv::Sampler (sampler.h:8-16): temperature / top-k / top-p sampling on host logits with a
+    std::minstd_rand0 stream; `seed=None` seeds from the random device as the reference does."""
+
+    def __init__(self, seed=None):
+        self._h = host()
+        self._s = self._h.fr_sampler_create(0 if seed is None else int(seed), 0 if seed is None else 1)
+        if not self._s:
+            raise FrhipError(self._h.fr_last_error().decode())
+
+    def set_seed(self, seed):
+        self._h.fr_sampler_set_seed(self._s, int(seed))
+
+    def sample(self, logits, temperature=1.0, top_k=0, top_p=1.0):
+        x = np.ascontiguousarray(logits, np.float32)
+        r = self._h.fr_sampler_sample(self._s, x.ctypes.data, x.size, temperature, top_k, top_p)
+        if r < 0:
+            raise FrhipError(self._h.fr_last_error().decode())
+        return r
+
+    def __del__(self):
+        if getattr(self, "_s", None):
+            self._h.fr_sampler_free(self._s)
+            self._s = None
 
 
 def write_fr(path, version, n_layer, n_embd, n_ffn, n_head, params, emb, quantized=None):

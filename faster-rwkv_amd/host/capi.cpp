@@ -9,6 +9,7 @@
 #include "kernels/hip/context.h"
 #include "kernels/kernels.h"
 #include "model.h"
+#include "sampler.h"
 
 namespace rwkv::hip {
 void allocator_stats(size_t *reserved, size_t *in_use, size_t *driver_calls);
@@ -93,6 +94,50 @@ long long fr_model_run_full(void *m, const int *ids, int n, float *logits, long 
     if (v > capacity) throw FRException("logits buffer too small");
     std::memcpy(logits, out.data_ptr<float>(), sizeof(float) * static_cast<size_t>(v));
     return v;
+  });
+}
+
+// Sampler (sampler.h:8-16).
+void *fr_sampler_create(int seed, int seeded) {
+  void *out = nullptr;
+  guarded([&]() {
+    auto *s = new rwkv::Sampler();
+    if (seeded) s->set_seed(seed);
+    out = s;
+    return 0;
+  });
+  return out;
+}
+
+void fr_sampler_free(void *s) { delete static_cast<rwkv::Sampler *>(s); }
+
+int fr_sampler_set_seed(void *s, int seed) {
+  return guarded([&]() {
+    static_cast<rwkv::Sampler *>(s)->set_seed(seed);
+    return 0;
+  });
+}
+
+// Sampler::Sample on a host buffer of n fp32 logits; returns the token id.
+int fr_sampler_sample(void *s, const float *logits, int n, float temperature, int top_k, float top_p) {
+  return guarded([&]() { return static_cast<rwkv::Sampler *>(s)->Sample(logits, n, temperature, top_k, top_p); });
+}
+
+// The generation loop of chat.cpp:56-92 without its penalties: feed first_id, sample, feed
+// the sample, `steps` times.  Returns the elapsed microseconds, or -1.
+long long fr_sample_decode(void *m, void *sampler, int first_id, int steps, float temperature, int top_k,
+                           float top_p, int *out_ids) {
+  return guarded([&]() -> long long {
+    auto *model = static_cast<rwkv::Model *>(m);
+    auto *smp = static_cast<rwkv::Sampler *>(sampler);
+    int id = first_id;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; i++) {
+      rwkv::Tensor out = model->Run(id);
+      id = smp->Sample(out, temperature, top_k, top_p);
+      out_ids[i] = id;
+    }
+    return std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count();
   });
 }
 

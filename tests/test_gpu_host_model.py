@@ -231,3 +231,21 @@ def test_full_output_gives_the_logits_of_every_position(model_files):
         lo = om.run(prompt[: t + 1]) if t else om.run(prompt[0])
         assert np.abs(full[t] - lo).max() <= 2e-2 and int(np.argmax(full[t])) == int(np.argmax(lo))
     m.close()
+
+
+def test_sampled_generation_follows_the_oracle_sampler(model_files):
+    """chat.cpp's loop with a seeded Sampler: the C++ loop on the hip model picks the tokens that the
+    sampler oracle picks from the same logits."""
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
+    import sampler_oracle as so
+    path, params, emb = model_files
+    m = fr.Model(path, "hip fp16")
+    toks, _ = m.generate(fr.Sampler(77), 5, 24, temperature=1.2, top_k=50, top_p=0.9)
+    m.reset()
+    g = so.MinStdRand0(77)
+    tok = 5
+    for i in range(24):
+        tok = so.sample(m.run(tok), 1.2, 50, 0.9, g)
+        assert tok == int(toks[i]), i
+    m.close()
