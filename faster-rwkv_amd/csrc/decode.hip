@@ -67,6 +67,7 @@ struct LnOut {
   bool active;
 };
 
+// `red` holds 2 * kWaves floats: the two reductions use separate halves, one barrier each.
 __device__ __forceinline__ LnOut ln_block(const h1* x, const h1* gamma, const h1* beta, int C, float* red) {
   const int e0 = threadIdx.x * 8;
   LnOut o;
@@ -84,7 +85,7 @@ __device__ __forceinline__ LnOut ln_block(const h1* x, const h1* gamma, const h1
       s += xf[i];
     }
   }
-  const float mean = block_sum<kWaves>(s, red) / (float)C;
+  const float mean = block_sum1<kWaves>(s, red) / (float)C;
   float q = 0.f;
   if (o.active) {
 #pragma unroll
@@ -93,7 +94,7 @@ __device__ __forceinline__ LnOut ln_block(const h1* x, const h1* gamma, const h1
       q += d * d;
     }
   }
-  float var = block_sum<kWaves>(q, red) / (float)C;
+  float var = block_sum1<kWaves>(q, red + kWaves) / (float)C;
   var = var > 0.f ? var : 0.f;
   const float inv = 1.0f / sqrtf(var + 1e-5f);
   if (o.active) {
@@ -140,8 +141,9 @@ struct RowBatch {
     }
   }
 
-  __device__ __forceinline__ void dot(const XVec (&xv)[R], const RowQ (&rq)[R], int nchunk, int lane,
-                                      float (&acc)[R]) const {
+  // Binary16 rows: acc[r] = sum_k w[k] x[k] against a binary16 vector.  uint8 rows:
+  // acc[r] = sum_k q[k] xr[k] against an fp32 vector staged by stage_q.
+  __device__ __forceinline__ void dot(const void* const (&xv)[R], int nchunk, int lane, float (&acc)[R]) const {
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
 #pragma unroll
@@ -151,31 +153,88 @@ struct RowBatch {
 #pragma unroll
         for (int r = 0; r < R; r++) {
           if constexpr (!U8) {
-            h8 x = reinterpret_cast<const h8*>(xv[r].x)[c];
+            h8 x = reinterpret_cast<const h8*>(xv[r])[c];
             acc[r] = dot8acc(w[r][j], x, acc[r]);
           } else {
-            // split staging: 8-element groups with even index first, odd ones second,
-            // so consecutive lanes read consecutive 16-byte LDS words
-            const h8* xp = reinterpret_cast<const h8*>(xv[r].x) + c;
-            const h8* ryp = reinterpret_cast<const h8*>(xv[r].ry) + c;
-            const h8* myp = reinterpret_cast<const h8*>(xv[r].my) + c;
-            const h2 c2 = {rq[r].c255, rq[r].c255};
-            const h2 m2 = {rq[r].mx, rq[r].mx};
+            const f32x4* xp = reinterpret_cast<const f32x4*>(xv[r]) + c;
+            float e = 0.f, o = 0.f;  // two chains per row so that consecutive fmas do not wait on each other
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) {
-              h8 x = xp[hh * nchunk], ry = ryp[hh * nchunk], my = myp[hh * nchunk];
-              uint32_t w0 = w[r][j][2 * hh], w1 = w[r][j][2 * hh + 1];
-              acc[r] = dot2acc(dequant_pair<0>(w0, c2, m2, ry.s01, my.s01), x.s01, acc[r]);
-              acc[r] = dot2acc(dequant_pair<1>(w0, c2, m2, ry.s23, my.s23), x.s23, acc[r]);
-              acc[r] = dot2acc(dequant_pair<0>(w1, c2, m2, ry.s45, my.s45), x.s45, acc[r]);
-              acc[r] = dot2acc(dequant_pair<1>(w1, c2, m2, ry.s67, my.s67), x.s67, acc[r]);
+            for (int jj = 0; jj < 4; jj++) {
+              const f32x4 x = xp[jj * nchunk];
+              const uint32_t word = w[r][j][jj];
+              e = __builtin_fmaf((float)(word & 0xffu), x[0], e);
+              o = __builtin_fmaf((float)((word >> 8) & 0xffu), x[1], o);
+              e = __builtin_fmaf((float)((word >> 16) & 0xffu), x[2], e);
+              o = __builtin_fmaf((float)(word >> 24), x[3], o);
             }
+            acc[r] += e + o;
           }
         }
       }
     }
   }
 };
+
+// ---------------------------------------------------------------------------
+// uint8 matrices in the row-streaming kernels.  With w^[n][k] = q c_n ry_k + mx_n + my_k
+// (c_n = rx_n / 255) a row's product factors into
+//   sum_k x_k w^[n][k] = c_n sum_k (x_k ry_k) q[n][k] + mx_n sum_k x_k + sum_k x_k my_k ,
+// so only the first sum depends on the row.  The workgroup stages xr_k = x_k ry_k in fp32 (the
+// product of two binary16 values is exact there) once per matrix and reduces Sx = sum x and
+// Smy = sum x my; a row then costs one byte-to-float conversion and one fma per code and
+// finishes as  c_n D_n + mx_n Sx + Smy.  This is the dequantisation formula evaluated in fp32
+// without its final rounding of w^ to binary16 (which the standalone dequantisation and the
+// matrix-matrix kernel apply); the difference is below the rounding of the binary16 output.
+//
+// xr is staged "split": a lane's chunk c covers 16 codes = four 16-byte groups of xr, and
+// group j of chunk c lives at f32x4 index j * nchunk + c, so that consecutive lanes read
+// consecutive 16-byte LDS words.
+// ---------------------------------------------------------------------------
+constexpr int kQSums = 2;  // Sx, Smy
+
+// Thread-owned group g = 8 consecutive elements of the vector.
+__device__ __forceinline__ void stage_q(float* dst, int g, int K, h8 x, h8 ry, h8 my, float* part) {
+  const int nchunk = K >> 4;
+  f32x4 lo, hi;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    lo[i] = (float)x[i] * (float)ry[i];
+    hi[i] = (float)x[4 + i] * (float)ry[4 + i];
+  }
+  const int c = g >> 1, j = (g & 1) * 2;
+  reinterpret_cast<f32x4*>(dst)[j * nchunk + c] = lo;
+  reinterpret_cast<f32x4*>(dst)[(j + 1) * nchunk + c] = hi;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    part[0] += (float)x[i];
+    part[1] += (float)x[i] * (float)my[i];
+  }
+}
+
+// Per-wave sums of the nval per-thread partials go to red[wave][v]; the caller's next barrier
+// publishes them, after which lane v of every wave gathers total v with gather_qsums.
+__device__ __forceinline__ void publish_qsums(const float* part, int nval, float (*red)[kMaxSeg * kQSums]) {
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  for (int v = 0; v < nval; v++) {
+    const float t = wave_sum(part[v]);
+    if (lane == 0) red[wv][v] = t;
+  }
+}
+
+__device__ __forceinline__ float gather_qsums(int nval, const float (*red)[kMaxSeg * kQSums]) {
+  const int lane = threadIdx.x & (kWave - 1);
+  float t = 0.f;
+  if (lane < nval) {
+#pragma unroll
+    for (int i = 0; i < kWaves; i++) t += red[i][lane];
+  }
+  return t;
+}
+
+__device__ __forceinline__ float finish_q(float d, float rx, float mx, float sx, float smy) {
+  const float c = rx / 255.0f;
+  return c * d + mx * sx + smy;
+}
 
 // ===========================================================================
 // att, front half:  LN -> mix -> k,v,r products -> sigmoid -> WKV-4 update
@@ -195,13 +254,15 @@ struct AttFrontV4 {
 template <int NCH, bool U8>
 __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ float red[kWaves];
+  __shared__ float red[2 * kWaves];
   const int C = a.C;
   const int nchunk = U8 ? (C >> 4) : (C >> 3);
-  h1* kx = reinterpret_cast<h1*>(smem);
-  h1* vx = kx + C;
-  h1* rx = vx + C;
-  h1* qv = rx + C;  // uint8 only: ry,my of kw ; ry,my of vw ; ry,my of rw
+  // binary16: the three mixed vectors; uint8: the three pre-scaled fp32 vectors xr (see stage_q)
+  constexpr int kElem = U8 ? 4 : 2;
+  unsigned char* kx = smem;
+  unsigned char* vx = kx + (size_t)kElem * C;
+  unsigned char* rx = vx + (size_t)kElem * C;
+  __shared__ float qred[kWaves][kMaxSeg * kQSums];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int gw = blockIdx.x * kWaves + threadIdx.x / kWave;
@@ -210,34 +271,56 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
 
   RowBatch<3, NCH, U8> cur;
-  // recurrent state and time parameters of the first channel, requested before anything else
   float st_tf = 0.f, st_td = 0.f, st_pp = 0.f, st_aa = 0.f, st_bb = 0.f;
   if (c0 < c1) {
     const void* rows[3] = {a.kw.data + c0 * row_bytes, a.vw.data + c0 * row_bytes, a.rw.data + c0 * row_bytes};
     cur.load(rows, nchunk, lane);
   }
 
+  // everything the prologue needs from global memory is requested before the layernorm's barriers
+  const bool own = (int)threadIdx.x * 8 < C;
+  const int e0 = threadIdx.x * 8;
+  h8 sx, mixk, mixv, mixr, qry[3], qmy[3];
+  if (own) {
+    sx = *reinterpret_cast<const h8*>(a.sx + e0);
+    mixk = *reinterpret_cast<const h8*>(a.mk + e0);
+    mixv = *reinterpret_cast<const h8*>(a.mv + e0);
+    mixr = *reinterpret_cast<const h8*>(a.mr + e0);
+    if constexpr (U8) {
+      qry[0] = *reinterpret_cast<const h8*>(a.kw.ry + e0); qmy[0] = *reinterpret_cast<const h8*>(a.kw.my + e0);
+      qry[1] = *reinterpret_cast<const h8*>(a.vw.ry + e0); qmy[1] = *reinterpret_cast<const h8*>(a.vw.my + e0);
+      qry[2] = *reinterpret_cast<const h8*>(a.rw.ry + e0); qmy[2] = *reinterpret_cast<const h8*>(a.rw.my + e0);
+    }
+  }
   LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, C, red);
+  float part[3 * kQSums];
+#pragma unroll
+  for (int i = 0; i < 3 * kQSums; i++) part[i] = 0.f;
   if (ln.active) {
-    const int e0 = threadIdx.x * 8;
-    h8 sx = *reinterpret_cast<const h8*>(a.sx + e0);
-    const int pos = stage_pos<U8>(threadIdx.x, C);
-    reinterpret_cast<h8*>(kx)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mk + e0));
-    reinterpret_cast<h8*>(vx)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mv + e0));
-    reinterpret_cast<h8*>(rx)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mr + e0));
+    const h8 mk = mix8(ln.xx, sx, mixk);
+    const h8 mv = mix8(ln.xx, sx, mixv);
+    const h8 mr = mix8(ln.xx, sx, mixr);
+    if constexpr (U8) {
+      stage_q(reinterpret_cast<float*>(kx), threadIdx.x, C, mk, qry[0], qmy[0], part + 0 * kQSums);
+      stage_q(reinterpret_cast<float*>(vx), threadIdx.x, C, mv, qry[1], qmy[1], part + 1 * kQSums);
+      stage_q(reinterpret_cast<float*>(rx), threadIdx.x, C, mr, qry[2], qmy[2], part + 2 * kQSums);
+    } else {
+      reinterpret_cast<h8*>(kx)[threadIdx.x] = mk;
+      reinterpret_cast<h8*>(vx)[threadIdx.x] = mv;
+      reinterpret_cast<h8*>(rx)[threadIdx.x] = mr;
+    }
     if (blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
   }
-  if constexpr (U8) {
-    stage_vec<true>(qv + 0 * C, a.kw.ry, C);
-    stage_vec<true>(qv + 1 * C, a.kw.my, C);
-    stage_vec<true>(qv + 2 * C, a.vw.ry, C);
-    stage_vec<true>(qv + 3 * C, a.vw.my, C);
-    stage_vec<true>(qv + 4 * C, a.rw.ry, C);
-    stage_vec<true>(qv + 5 * C, a.rw.my, C);
-  }
+  if constexpr (U8) publish_qsums(part, 3 * kQSums, qred);
   __syncthreads();
+  float qt[3 * kQSums];
+  if constexpr (U8) {
+    const float tv = gather_qsums(3 * kQSums, qred);
+#pragma unroll
+    for (int i = 0; i < 3 * kQSums; i++) qt[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tv), i));
+  }
 
-  const XVec xv[3] = {{kx, qv + 0 * C, qv + 1 * C}, {vx, qv + 2 * C, qv + 3 * C}, {rx, qv + 4 * C, qv + 5 * C}};
+  const void* const xv[3] = {kx, vx, rx};
   for (int n = c0; n < c1; n++) {
     RowBatch<3, NCH, U8> nxt;
     if (n + 1 < c1) {
@@ -245,17 +328,16 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
                              a.rw.data + (n + 1) * row_bytes};
       nxt.load(rows, nchunk, lane);
     }
-    RowQ rq[3];
-    if constexpr (U8) {
-      rq[0] = {dequant_c255(a.kw.rx[n]), a.kw.mx[n]};
-      rq[1] = {dequant_c255(a.vw.rx[n]), a.vw.mx[n]};
-      rq[2] = {dequant_c255(a.rw.rx[n]), a.rw.mx[n]};
-    }
     float acc[3];
-    cur.dot(xv, rq, nchunk, lane, acc);
-    const float k = wave_sum(acc[0]);
-    const float v = wave_sum(acc[1]);
-    const float rr = wave_sum(acc[2]);
+    cur.dot(xv, nchunk, lane, acc);
+    float k = wave_sum(acc[0]);
+    float v = wave_sum(acc[1]);
+    float rr = wave_sum(acc[2]);
+    if constexpr (U8) {
+      k = finish_q(k, (float)a.kw.rx[n], (float)a.kw.mx[n], qt[0], qt[1]);
+      v = finish_q(v, (float)a.vw.rx[n], (float)a.vw.mx[n], qt[2], qt[3]);
+      rr = finish_q(rr, (float)a.rw.rx[n], (float)a.rw.mx[n], qt[4], qt[5]);
+    }
     if (lane == 0) {
       // kernels/cuda/att.cu:30-62 (WkvForwardOne), r already passed through sigmoid (:203)
       {
@@ -356,12 +438,15 @@ __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, i
 template <int R, int NCH, bool U8, bool MULTI>
 __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ float red[kWaves];
+  __shared__ float red[2 * kWaves];
   const int K = a.K;
   const int nchunk = U8 ? (K >> 4) : (K >> 3);
   const size_t row_bytes = U8 ? (size_t)K : 2 * (size_t)K;
-  h1* vecs = reinterpret_cast<h1*>(smem);   // nvec staged activation vectors
-  h1* qv = vecs + (size_t)a.nvec * K;       // uint8: (ry, my) per segment
+  // binary16: nvec staged activation vectors; uint8: one pre-scaled fp32 vector xr per segment
+  h1* vecs = reinterpret_cast<h1*>(smem);
+  float* qvecs = reinterpret_cast<float*>(smem);
+  __shared__ float qred[kWaves][kMaxSeg * kQSums];
+  float qtv = 0.f;  // uint8: lane v holds total v of (Sx, Smy) x segments
 
   const int lane = threadIdx.x & (kWave - 1);
   // The concatenated row space of all segments is split evenly over the waves of the grid;
@@ -391,21 +476,16 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     m.er = (h1)0.0f;
   };
   auto consume = [&](const RowBatch<R, NCH, U8>& b, const Meta& m, int g) {
-    XVec xv[R];
-    RowQ rq[R];
+    const void* xv[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const Seg& sg = a.seg[m.seg[r]];
-      xv[r].x = vecs + (size_t)sg.vec * K;
-      xv[r].ry = qv + (size_t)(2 * m.seg[r]) * K;
-      xv[r].my = qv + (size_t)(2 * m.seg[r] + 1) * K;
-      if constexpr (U8) {
-        rq[r].c255 = dequant_c255(sg.w.rx[m.loc[r]]);
-        rq[r].mx = sg.w.mx[m.loc[r]];
-      }
+      if constexpr (U8)
+        xv[r] = qvecs + (size_t)m.seg[r] * K;
+      else
+        xv[r] = vecs + (size_t)a.seg[m.seg[r]].vec * K;
     }
     float acc[R];
-    b.dot(xv, rq, nchunk, lane, acc);
+    b.dot(xv, nchunk, lane, acc);
     float mine = 0.f;
     int my_seg = 0, my_loc = 0;
 #pragma unroll
@@ -417,7 +497,18 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
         my_loc = m.loc[r];
       }
     }
-    if (lane < R && g + lane < g1) run_epilogue(a, a.seg[my_seg], my_loc, mine, m.ex, m.er);
+    float q0 = 0.f, q1 = 0.f;
+    if constexpr (U8) {  // lane v holds total v: fetch the two of this lane's segment (all lanes take part)
+      q0 = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (my_seg * kQSums + 0), __float_as_int(qtv)));
+      q1 = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (my_seg * kQSums + 1), __float_as_int(qtv)));
+    }
+    if (lane < R && g + lane < g1) {
+      if constexpr (U8) {
+        const WMat& w = a.seg[my_seg].w;
+        mine = finish_q(mine, (float)w.rx[my_loc], (float)w.mx[my_loc], q0, q1);
+      }
+      run_epilogue(a, a.seg[my_seg], my_loc, mine, m.ex, m.er);
+    }
   };
 
   RowBatch<R, NCH, U8> A;
@@ -425,30 +516,78 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   if (g0 < g1) fetch(A, mA, g0);
 
   // ---- prologue: stage the activation vector(s) in LDS ----
-  if (a.prologue == P_COPY) {
-    stage_vec<U8>(vecs, a.vec0, K);
-  } else {
-    LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, K, red);
-    if (ln.active) {
-      const int e0 = threadIdx.x * 8;
-      const int pos = stage_pos<U8>(threadIdx.x, K);
-      if (a.prologue == P_LN) {
-        reinterpret_cast<h8*>(vecs)[pos] = ln.xx;
-      } else {
-        h8 sx = *reinterpret_cast<const h8*>(a.sx + e0);
-        for (int i = 0; i < a.nvec; i++)
-          reinterpret_cast<h8*>(vecs + (size_t)i * K)[pos] = mix8(ln.xx, sx, *reinterpret_cast<const h8*>(a.mix[i] + e0));
-        if (blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
+  // Global operands of the prologue are requested before the layernorm's barriers.
+  {
+    const int e0 = threadIdx.x * 8;
+    const bool own = a.prologue != P_COPY && e0 < K;
+    h8 sx, mixv[kMaxSeg], qry[kMaxSeg], qmy[kMaxSeg];
+    if (own) {
+      if (a.prologue == P_LN_MIX) {
+        sx = *reinterpret_cast<const h8*>(a.sx + e0);
+#pragma unroll
+        for (int i = 0; i < kMaxSeg; i++)
+          if (i < a.nvec) mixv[i] = *reinterpret_cast<const h8*>(a.mix[i] + e0);
+      }
+      if constexpr (U8) {
+#pragma unroll
+        for (int i = 0; i < kMaxSeg; i++)
+          if (i < a.nseg) {
+            qry[i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + e0);
+            qmy[i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + e0);
+          }
       }
     }
-  }
-  if constexpr (U8) {
-    for (int s = 0; s < a.nseg; s++) {
-      stage_vec<true>(qv + (size_t)(2 * s) * K, a.seg[s].w.ry, K);
-      stage_vec<true>(qv + (size_t)(2 * s + 1) * K, a.seg[s].w.my, K);
+    float part[kMaxSeg * kQSums];
+#pragma unroll
+    for (int i = 0; i < kMaxSeg * kQSums; i++) part[i] = 0.f;
+    if (a.prologue == P_COPY) {
+      if constexpr (!U8) {
+        stage_vec<false>(vecs, a.vec0, K);
+      } else {
+        for (int g = threadIdx.x; g < (K >> 3); g += kThreads) {
+          const h8 x = reinterpret_cast<const h8*>(a.vec0)[g];
+#pragma unroll
+          for (int i = 0; i < kMaxSeg; i++)
+            if (i < a.nseg)
+              stage_q(qvecs + (size_t)i * K, g, K, x, *reinterpret_cast<const h8*>(a.seg[i].w.ry + 8 * g),
+                      *reinterpret_cast<const h8*>(a.seg[i].w.my + 8 * g), part + i * kQSums);
+        }
+      }
+    } else {
+      LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, K, red);
+      if (ln.active) {
+        if constexpr (!U8) {
+          if (a.prologue == P_LN) {
+            reinterpret_cast<h8*>(vecs)[threadIdx.x] = ln.xx;
+          } else {
+#pragma unroll
+            for (int i = 0; i < kMaxSeg; i++)
+              if (i < a.nvec) reinterpret_cast<h8*>(vecs + (size_t)i * K)[threadIdx.x] = mix8(ln.xx, sx, mixv[i]);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < kMaxSeg; i++) {
+            if (i < a.nseg) {
+              h8 x = ln.xx;
+              if (a.prologue == P_LN_MIX) {
+                // segment i multiplies staged vector seg[i].vec; pick its mix without dynamic register indexing
+                h8 mx8 = mixv[0];
+#pragma unroll
+                for (int j = 1; j < kMaxSeg; j++)
+                  if (a.seg[i].vec == j) mx8 = mixv[j];
+                x = mix8(ln.xx, sx, mx8);
+              }
+              stage_q(qvecs + (size_t)i * K, threadIdx.x, K, x, qry[i], qmy[i], part + i * kQSums);
+            }
+          }
+        }
+        if (a.prologue == P_LN_MIX && blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
+      }
     }
+    if constexpr (U8) publish_qsums(part, a.nseg * kQSums, qred);
+    __syncthreads();
+    if constexpr (U8) qtv = gather_qsums(a.nseg * kQSums, qred);
   }
-  __syncthreads();
 
   if constexpr (!MULTI) {
     if (g0 < g1) consume(A, mA, g0);  // the host guarantees g1 - g0 <= R
@@ -665,7 +804,7 @@ static int launch_rows(const RowsArgs& a, bool u8, hipStream_t st, const char* w
   const int grid = decode_grid();
   bool multi = false;
   const int R = pick_r(a, grid, nch, u8, &multi);
-  const size_t lds = 2 * (size_t)a.K * (a.nvec + (u8 ? 2 * a.nseg : 0));
+  const size_t lds = u8 ? 4 * (size_t)a.K * a.nseg : 2 * (size_t)a.K * a.nvec;
   FR_TRY(check_lds(lds));
   bool ok = false;
   switch (nch) {
@@ -781,7 +920,7 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   a.xx_out = (h1*)xx_out; a.rwkv_out = w.rwkv;
   a.aa_out = aa_out; a.bb_out = bb_out; a.pp_out = pp_out;
   const bool u8 = kw->dtype == FRHIP_U8;
-  const size_t lds = 2 * (size_t)C * (u8 ? 9 : 3);
+  const size_t lds = (u8 ? 4 : 2) * (size_t)C * 3;
   FR_TRY(check_lds(lds));
   const int nch = chunks_per_lane(C, u8);  // C <= 4096: at most 8 (fp16) or 4 (uint8)
 #define FR_ATT_FRONT(N)                                                                                   \

@@ -99,10 +99,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
         int row = n0 + (c >> 2);
         row = row < N ? row : N - 1;
         const int kk = k0 + (c & 3) * 16;
-        const h1 c255 = dequant_c255(sg.rx[row]);
-        const h2 c2 = {c255, c255};
-        const h1 mxv = sg.mx[row];
-        const h2 m2 = {mxv, mxv};
+        const float c2 = dequant_c(sg.rx[row]);
+        const float m2 = (float)sg.mx[row];
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
           const h8 ry = *reinterpret_cast<const h8*>(sg.ry + kk + hh * 8);

@@ -132,9 +132,8 @@ __global__ void dequant_u8_kernel(const uint32_t* __restrict__ q, const h1* __re
   if (i >= words) return;
   const int n = (int)(i / (K >> 2));
   const int k = (int)(i % (K >> 2)) * 4;
-  const h1 c = dequant_c255(rx[n]);
-  const h2 c2 = {c, c};
-  const h2 m2 = {mx[n], mx[n]};
+  const float c2 = dequant_c(rx[n]);
+  const float m2 = (float)mx[n];
   const uint32_t w = q[i];
   h2 ry01 = {ry[k], ry[k + 1]}, ry23 = {ry[k + 2], ry[k + 3]};
   h2 my01 = {my[k], my[k + 1]}, my23 = {my[k + 2], my[k + 3]};

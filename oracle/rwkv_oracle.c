@@ -330,26 +330,18 @@ static void wkv4_one_f32(const float *t_first, const float *t_decay, const float
 /* ======================================================================== */
 
 orc_half orc_dequant_u8_scalar(uint8_t q, orc_half mx, orc_half rx, orc_half my, orc_half ry) {
-  const orc_half h255 = 0x5BF8; /* 255.0 */
-  orc_half c255 = orc_hdiv(rx, h255);
-  orc_half a = orc_hmul(c255, ry);
-  orc_half b = orc_hadd(mx, my);
-  return orc_hfma(orc_f2h((float)q), a, b);
+  float c = orc_h2f(rx) / 255.0f;
+  float a = c * orc_h2f(ry);
+  float b = orc_h2f(mx) + orc_h2f(my);
+  return orc_f2h(fmaf((float)q, a, b));
 }
 
 void orc_dequant_u8(const uint8_t *q, const orc_half *mx, const orc_half *rx,
                     const orc_half *my, const orc_half *ry, orc_half *W, int K, int N) {
-  const orc_half h255 = 0x5BF8;
-  orc_half *c255 = (orc_half *)xmalloc(sizeof(orc_half) * (size_t)N);
-  for (int n = 0; n < N; n++) c255[n] = orc_hdiv(rx[n], h255);
 #pragma omp parallel for schedule(static)
   for (int k = 0; k < K; k++)
-    for (int n = 0; n < N; n++) {
-      orc_half a = orc_hmul(c255[n], ry[k]);
-      orc_half b = orc_hadd(mx[n], my[k]);
-      W[(size_t)k * N + n] = orc_hfma(orc_f2h((float)q[(size_t)k * N + n]), a, b);
-    }
-  free(c255);
+    for (int n = 0; n < N; n++)
+      W[(size_t)k * N + n] = orc_dequant_u8_scalar(q[(size_t)k * N + n], mx[n], rx[n], my[k], ry[k]);
 }
 
 /* ======================================================================== */

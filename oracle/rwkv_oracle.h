@@ -21,7 +21,7 @@
  * The uint8 dequantisation formula has no counterpart in the reference tree
  * (kernels/kernels.h:11-13 only names the mx/rx/my/ry parameters): PARITY UNPINNED
  * by the reference; it is pinned here by exhaustive evaluation against an
- * independent numpy-float16 statement of the same formula.
+ * independent numpy statement of the same formula.
  */
 #ifndef RWKV_ORACLE_H_
 #define RWKV_ORACLE_H_
@@ -82,11 +82,13 @@ void orc_wkv4_one_f16(const float *t_first, const float *t_decay, const float *k
                       const float *v, float *aa, float *bb, float *pp, orc_half *r, int n);
 
 /* ---- uint8 weight-only quantisation (ChatRWKV-style mx/rx/my/ry) ---------- */
-/* Dequantised weight, all operations in binary16 with RTNE:
- *     c255 = h(rx[n] / h(255))          (per output column n)
- *     a    = h(c255 * ry[k])            (per element)
- *     b    = h(mx[n] + my[k])
- *     w^   = h(fma(h(q), a, b))         (single rounding)
+/* Dequantised weight, evaluated in IEEE binary32 with one final RTNE to binary16:
+ *     c  = f32(rx[n]) / 255             (per output column n)
+ *     a  = c * f32(ry[k])               (per element)
+ *     b  = f32(mx[n]) + f32(my[k])
+ *     w^ = h(fmaf(q, a, b))
+ * (binary16 intermediates would put a relative error of 2^-12 on c, the same for a whole
+ * column, which a product with same-signed activations does not average out.)
  * q is [K,N] row-major, mx,rx are [N] (per column), my,ry are [K] (per row). */
 orc_half orc_dequant_u8_scalar(uint8_t q, orc_half mx, orc_half rx, orc_half my, orc_half ry);
 void orc_dequant_u8(const uint8_t *q, const orc_half *mx, const orc_half *rx,

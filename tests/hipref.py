@@ -53,7 +53,12 @@ def make_weight(w_kn, quant=False):
     import pyoracle as po
     from synth import quantize_u8
     q, mx, rx, my, ry = quantize_u8(w_kn)
-    return PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry), po.dequant_u8(q, mx, rx, my, ry)
+    pw = PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry)
+    f = np.float64
+    # the real-valued formula the codes stand for, before any rounding of w^
+    pw.exact = lambda: (q.astype(f) * (rx.astype(f) / 255)[None, :] * ry.astype(f)[:, None]
+                        + mx.astype(f)[None, :] + my.astype(f)[:, None])
+    return pw, po.dequant_u8(q, mx, rx, my, ry)
 
 
 class HipModelV4:

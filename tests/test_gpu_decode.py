@@ -62,9 +62,11 @@ def test_att_one_v4(C_, quant, fresh_state):
                                   ws[0].ref, ws[1].ref, ws[2].ref, ws[3].ref, x_out.ptr, xx_out.ptr,
                                   aa_o.ptr, bb_o.ptr, pp_o.ptr, wsb.ptr, None))
     assert_close_f16(xx_out.numpy(), ref[1], max_ulp=1, what="xx")
-    assert_close_f16(x_out.numpy(), ref[0], max_ulp=2, what="x_out")
+    # uint8: the kernels multiply by w^ before its rounding to binary16, the oracle after it:
+    # more one-spacing flips, same bound on their size
+    assert_close_f16(x_out.numpy(), ref[0], max_ulp=2, max_frac=0.3 if quant else 0.03, what="x_out")
     for got, want, nm in ((aa_o, ref[2], "aa"), (bb_o, ref[3], "bb"), (pp_o, ref[4], "pp")):
-        assert np.allclose(got.numpy(), want, rtol=2e-4, atol=2e-5), nm
+        assert np.allclose(got.numpy(), want, rtol=2e-4, atol=(2e-3 * np.abs(want).max()) if quant else 2e-5), nm
 
 
 @pytest.mark.parametrize("C_,F_", [(2048, 8192), (768, 3072), (512, 1024)])
@@ -87,7 +89,7 @@ def test_ffn_one(C_, F_, quant, div2):
     assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx")
     # A one-spacing flip in a few of the F relu^2 values moves many of the C outputs of
     # the last product by one spacing, so the end-to-end comparison is loose ...
-    assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
+    assert_close_f16(x_out.numpy(), ref_x, max_ulp=4 if quant else 3, max_frac=0.5 if quant else 0.2, what="x_out")
     # ... and the strict one restarts the oracle from the kernel's own intermediates
     # (workspace: binary16 rwkv | r | x_mid | g, fp32 k | v | r32, binary16 vx; each rounded up
     # to 256 bytes): bit-exact.
@@ -97,8 +99,17 @@ def test_ffn_one(C_, F_, quant, div2):
     vx_g = ws[(4 * al(2 * C_) + 3 * al(4 * C_)) // 2:][:F_]
     r_ref = po.sigmoid_f16(po.gemm_f16(po.mix_f16(ref_xx, sx, mr), rref, "f16"))
     vx_ref = po.relu_square_f16(po.gemm_f16(po.mix_f16(ref_xx, sx, mk), kref, "f16"))
-    assert_close_f16(r_g, r_ref, max_ulp=1, max_frac=0.01, what="r")
-    assert_close_f16(vx_g, vx_ref, max_ulp=3, max_frac=0.01, what="vx")  # a one-spacing flip of t becomes up to three in t*t
+    assert_close_f16(r_g, r_ref, max_ulp=2 if quant else 1, max_frac=0.1 if quant else 0.01, what="r")
+    assert_close_f16(vx_g, vx_ref, max_ulp=6 if quant else 3, max_frac=0.3 if quant else 0.01, what="vx")  # a one-spacing flip of t becomes up to three in t*t
+    if quant:
+        # the last product against the real-valued weights, from the kernel's own r and vx
+        out_e = (vx_g.astype(np.float64) @ vw.exact()).astype(np.float16)
+        strict = np.array([po.lib.orc_hfma(int(a), int(b), int(c)) for a, b, c in
+                           zip(out_e.view(np.uint16), r_g.view(np.uint16), x.view(np.uint16))], np.uint16).view(np.float16)
+        if div2:
+            strict = (strict.astype(np.float32) / 2).astype(np.float16)
+        assert_close_f16(x_out.numpy(), strict, max_ulp=2, max_frac=0.01, what="x_out from kernel intermediates (uint8)")
+        return
     out_g = po.gemm_f16(vx_g, vref, "f16")
     strict = np.array([po.lib.orc_hfma(int(a), int(b), int(c)) for a, b, c in
                        zip(out_g.view(np.uint16), r_g.view(np.uint16), x.view(np.uint16))], np.uint16).view(np.float16)
@@ -134,10 +145,10 @@ def test_att_one_v5_1(C_, H_, quant):
                                     keep(tf).ptr, *[w.ref for w in ws], x_out.ptr, xx_out.ptr, s_out.ptr, wsb.ptr,
                                     None))
     assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx")
-    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-5, atol=1e-5)
+    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-5, atol=2e-3 if quant else 1e-5)
     # groupnorm amplifies the fp32 summation-order noise of the head outputs; a few one-spacing
     # flips of the gated vector then spread over the output product
-    assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
+    assert_close_f16(x_out.numpy(), ref_x, max_ulp=5 if quant else 3, max_frac=0.4 if quant else 0.2, what="x_out")
 
 
 @pytest.mark.parametrize("C_,H_", [(2048, 32), (512, 8)])
@@ -167,8 +178,8 @@ def test_att_one_v5(C_, H_, quant):
                                   keep(tf).ptr, *[w.ref for w in ws], x_out.ptr, xx_out.ptr, s_out.ptr, wsb.ptr,
                                   None))
     assert_close_f16(xx_out.numpy(), ref_xx, max_ulp=1, what="xx")
-    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-5, atol=1e-5)
-    assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out")
+    assert np.allclose(s_out.numpy(), ref_s, rtol=1e-5, atol=2e-3 if quant else 1e-5)
+    assert_close_f16(x_out.numpy(), ref_x, max_ulp=5 if quant else 3, max_frac=0.4 if quant else 0.2, what="x_out")
 
 
 @pytest.mark.parametrize("quant", [False, True])
@@ -182,7 +193,12 @@ def test_head(quant):
     fr.check(L().frhip_head(C_, keep(x).ptr, keep(ln_w).ptr, keep(ln_b).ptr, hw.ref, out.ptr, None))
     got = out.numpy()
     assert np.abs(got - ref).max() <= 2e-2
-    assert_close_f16(got.astype(np.float16), ref.astype(np.float16), max_ulp=2, max_frac=0.05, what="logits")
+    if quant:  # tight against the real-valued weights, loose against the oracle's binary16 w^
+        exact = po.layernorm_f16(x, ln_w, ln_b).astype(np.float64) @ hw.exact()
+        assert_close_f16(got.astype(np.float16), exact.astype(np.float16), max_ulp=1, max_frac=0.01, what="logits vs real-valued weights")
+        assert np.abs(got - ref).max() <= 4e-3
+    else:
+        assert_close_f16(got.astype(np.float16), ref.astype(np.float16), max_ulp=2, max_frac=0.05, what="logits")
 
 
 def _greedy_pair(L_, C_, F_, V_, quant, steps, seed):

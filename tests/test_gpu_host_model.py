@@ -25,6 +25,13 @@ def model_files(tmp_path_factory):
     return path, params, emb
 
 
+def _same_token(lh, lo):
+    """Greedy tokens agree, or the oracle's own margin between the two candidates is a tie at the
+    resolution of binary16 logits (one spacing near 1.0 is 9.8e-4)."""
+    a, b = int(np.argmax(lh)), int(np.argmax(lo))
+    return a == b or float(lo[b] - lo[a]) <= 1e-3
+
+
 def _oracle(params, emb, quant):
     p = list(params)
     if quant:
@@ -152,7 +159,10 @@ def test_rwkv5_2_model_matches_oracle(tmp_path):
         for step in range(64):
             lh, lo = m.run(tok), om.run(tok)
             worst = max(worst, float(np.abs(lh - lo).max()))
-            assert int(np.argmax(lh)) == int(np.argmax(lo)), "greedy token differs at step %d" % step
+            if int(np.argmax(lh)) != int(np.argmax(lo)):
+                # only a tie at the resolution of binary16 logits (one spacing near 1.0 is 9.8e-4) may differ
+                margin = float(lo.max() - lo[int(np.argmax(lh))])
+                assert margin <= 1e-3, "greedy token differs at step %d (oracle margin %g)" % (step, margin)
             tok = int(np.argmax(lo))
         print(strategy, "v5.2 worst |dlogit| over 64 steps:", worst, flush=True)
         assert worst <= 2e-2
@@ -164,7 +174,7 @@ def test_rwkv5_2_model_matches_oracle(tmp_path):
         om.reset()
         prompt = [int(t) for t in np.random.default_rng(44).integers(0, V5, 96)]
         ls, lo = m.run(prompt), om.run(prompt)
-        assert np.abs(ls - lo).max() <= 2e-2 and int(np.argmax(ls)) == int(np.argmax(lo))
+        assert np.abs(ls - lo).max() <= 2e-2 and _same_token(ls, lo)
         tok = int(np.argmax(lo))
         for step in range(8):
             ls, lo = m.run(tok), om.run(tok)
@@ -205,7 +215,7 @@ def test_rwkv5_0_model_matches_oracle(tmp_path):
         om.reset()
         prompt = [int(t) for t in np.random.default_rng(45).integers(0, V5, 80)]
         ls, lo = m.run(prompt), om.run(prompt)
-        assert np.abs(ls - lo).max() <= 2e-2 and int(np.argmax(ls)) == int(np.argmax(lo))
+        assert np.abs(ls - lo).max() <= 2e-2 and _same_token(ls, lo)
         tok = int(np.argmax(lo))
         for step in range(8):
             ls, lo = m.run(tok), om.run(tok)

@@ -98,14 +98,17 @@ def test_dequant_all_codes_bit_exact():
         out = DevBuf.empty((N, K), np.float16)
         fr.check(L().frhip_dequant_u8(w.ref, out.ptr, None))
         assert np.array_equal(out.numpy().T.view(np.uint16), ref.view(np.uint16))
-        # the dequantisation fused into the matrix-vector kernel: a one-hot activation
-        # returns row k of the dequantised matrix exactly (fp32 output, 1*w + 0's)
+        # the matrix-vector kernel evaluates the same formula in fp32 without the final rounding of
+        # w^ to binary16: a one-hot activation returns q c ry + mx + my of row k to fp32 accuracy
         y = DevBuf.empty(N, np.float32)
+        f = np.float64
         for k in (0, 1, 17, 200, 255):
             e = np.zeros(K, np.float16)
             e[k] = 1
             fr.check(L().frhip_gemv(keep(e).ptr, w.ref, y.ptr, fr.F32, None))
-            assert np.array_equal(y.numpy(), ref[k].astype(np.float32)), k
+            terms = (np.abs(q[k].astype(f) * (rx.astype(f) / 255) * f(ry[k])), np.abs(mx.astype(f)), abs(f(my[k])))
+            exact = q[k].astype(f) * (rx.astype(f) / 255) * f(ry[k]) + mx.astype(f) + f(my[k])
+            assert (np.abs(y.numpy() - exact) <= 4e-7 * (terms[0] + terms[1] + terms[2]) + 1e-30).all(), k
 
 
 def test_dequant_random_matrix_bit_exact():
@@ -132,8 +135,23 @@ def test_gemv_against_oracle(K, N, quant):
     fr.check(L().frhip_gemv(keep(x).ptr, pw.ref, y32.ptr, fr.F32, None))
     fr.check(L().frhip_gemv(keep(x).ptr, pw.ref, y16.ptr, fr.F16, None))
     tol = 2e-6 * np.sqrt(K) * np.abs(ref32).max() + 1e-6
-    assert np.abs(y32.numpy() - ref32).max() <= tol + 2e-5
-    assert_close_f16(y16.numpy(), ref32.astype(np.float16), max_ulp=1, what="gemv f16 out")
+    if not quant:
+        assert np.abs(y32.numpy() - ref32).max() <= tol + 2e-5
+        assert_close_f16(y16.numpy(), ref32.astype(np.float16), max_ulp=1, what="gemv f16 out")
+        return
+    # uint8: the kernel evaluates sum_k x_k (q c ry + mx + my) in fp32 without rounding w^ to
+    # binary16 -> tight against the real-valued formula in float64 ...
+    exact = x.astype(np.float64) @ pw.exact()
+    mag = np.abs(x.astype(np.float64)) @ np.abs(pw.exact())
+    assert (np.abs(y32.numpy() - exact) <= 4e-6 * mag + 1e-6).all()
+    # ... and within the w^-rounding noise of the oracle, which multiplies by binary16 w^
+    # (relative error up to 2^-12 per element, uniform): six standard deviations of that sum
+    rms = lambda a: float(np.sqrt(np.mean(np.asarray(a, np.float64) ** 2)))
+    noise = 6 * (2.0 ** -12 / np.sqrt(3)) * np.sqrt(K) * rms(x) * rms(wref)
+    assert np.abs(y32.numpy() - ref32).max() <= tol + noise + 2e-5
+    r16 = ref32.astype(np.float16).astype(np.float32)
+    half_spacing = np.exp2(np.floor(np.log2(np.maximum(np.abs(r16), 1e-7))) - 11)
+    assert (np.abs(y16.numpy().astype(np.float32) - r16) <= noise + 2 * half_spacing).all()
 
 
 def test_gemv_rejects_bad_arguments():

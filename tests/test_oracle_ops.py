@@ -274,14 +274,17 @@ def test_att_v5_0_seq_equals_loop_of_one_token_steps():
 
 # ---------------------------------------------------------------- dequant u8
 def _dequant_numpy(q, mx, rx, my, ry):
-    """Independent numpy-float16 statement of the dequantisation: every operation in
-    binary16; the fused multiply-add done exactly in float64 (exact for these operands)."""
-    c255 = (rx / np.float16(255)).astype(np.float16)
-    a = (c255[None, :] * ry[:, None]).astype(np.float16)
-    b = (mx[None, :] + my[:, None]).astype(np.float16)
-    # q*a has <= 19 significant bits and |exponent gap| to b is small: float64 sum is exact
-    exact = q.astype(np.float64) * a.astype(np.float64) + b.astype(np.float64)
-    return exact.astype(np.float16)  # float64 -> float16 in numpy is a single RTNE rounding
+    """Independent numpy statement of the dequantisation: c = rx/255, a = c*ry, b = mx+my in
+    float32 (numpy's float32 operations are correctly rounded), the fused multiply-add exactly
+    in the 64-bit-mantissa long double (q*a has <= 32 significant bits; the widest exponent gap
+    to b on the grid below is 2^27), then one rounding to float32 and one to float16."""
+    assert np.finfo(np.longdouble).nmant >= 63
+    f = np.float32
+    c = rx.astype(f) / f(255)
+    a = c[None, :] * ry.astype(f)[:, None]
+    b = mx.astype(f)[None, :] + my.astype(f)[:, None]
+    exact = q.astype(np.longdouble) * a.astype(np.longdouble) + b.astype(np.longdouble)
+    return exact.astype(f).astype(np.float16)
 
 
 def test_dequant_all_codes_times_scale_grid_bit_exact():
