@@ -124,10 +124,15 @@ __device__ __forceinline__ void split_even(int total, int parts, int i, int& lo,
 // A batch of R weight rows held in registers: NCH 16-byte chunks per lane per row
 // (lane l owns chunks l, l+64, ...).  load() only issues the loads; dot() consumes
 // them against LDS-resident vectors.  K <= NCH * 64 * (8 | 16) elements.
+// Neither contains a branch, so that the compiler can count the loads in flight and let
+// dot() start on the first chunk while later ones (and the next batch) are still on their
+// way: a lane whose chunk index lies beyond the row re-reads the row's last chunk, and the
+// staged vectors are padded with zeros up to NCH * 64 chunks, which cancels it.
 // ---------------------------------------------------------------------------
 template <int R, int NCH, bool U8>
 struct RowBatch {
   using V = typename std::conditional<U8, u32x4, h8>::type;
+  static constexpr int kPadChunks = NCH * kWave;  // chunks per staged vector, padding included
   V w[R][NCH];
 
   __device__ __forceinline__ void load(const void* const (&rows)[R], int nchunk, int lane) {
@@ -135,45 +140,94 @@ struct RowBatch {
     for (int r = 0; r < R; r++) {
 #pragma unroll
       for (int j = 0; j < NCH; j++) {
-        const int c = lane + j * kWave;
-        if (c < nchunk) w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const V*>(rows[r]) + c);
+        int c = lane + j * kWave;
+        c = c < nchunk ? c : nchunk - 1;
+        w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const V*>(rows[r]) + c);
+      }
+    }
+  }
+
+  // All rows against the same staged vector: each chunk of it is read from LDS once.
+  __device__ __forceinline__ void dot_shared(const void* xv, int lane, float (&acc)[R]) const {
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+      const int c = lane + j * kWave;
+      if constexpr (!U8) {
+        const h8 x = reinterpret_cast<const h8*>(xv)[c];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = dot8acc(w[r][j], x, acc[r]);
+      } else {
+        const f32x4* xp = reinterpret_cast<const f32x4*>(xv) + c;
+        float e[R], o[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) e[r] = o[r] = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+          const f32x4 x = xp[jj * kPadChunks];
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+            const uint32_t word = w[r][j][jj];
+            e[r] = __builtin_fmaf((float)(word & 0xffu), x[0], e[r]);
+            o[r] = __builtin_fmaf((float)((word >> 8) & 0xffu), x[1], o[r]);
+            e[r] = __builtin_fmaf((float)((word >> 16) & 0xffu), x[2], e[r]);
+            o[r] = __builtin_fmaf((float)(word >> 24), x[3], o[r]);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += e[r] + o[r];
       }
     }
   }
 
   // Binary16 rows: acc[r] = sum_k w[k] x[k] against a binary16 vector.  uint8 rows:
   // acc[r] = sum_k q[k] xr[k] against an fp32 vector staged by stage_q.
-  __device__ __forceinline__ void dot(const void* const (&xv)[R], int nchunk, int lane, float (&acc)[R]) const {
+  __device__ __forceinline__ void dot(const void* const (&xv)[R], int lane, float (&acc)[R]) const {
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
       const int c = lane + j * kWave;
-      if (c < nchunk) {
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-          if constexpr (!U8) {
-            h8 x = reinterpret_cast<const h8*>(xv[r])[c];
-            acc[r] = dot8acc(w[r][j], x, acc[r]);
-          } else {
-            const f32x4* xp = reinterpret_cast<const f32x4*>(xv[r]) + c;
-            float e = 0.f, o = 0.f;  // two chains per row so that consecutive fmas do not wait on each other
+      for (int r = 0; r < R; r++) {
+        if constexpr (!U8) {
+          h8 x = reinterpret_cast<const h8*>(xv[r])[c];
+          acc[r] = dot8acc(w[r][j], x, acc[r]);
+        } else {
+          const f32x4* xp = reinterpret_cast<const f32x4*>(xv[r]) + c;
+          float e = 0.f, o = 0.f;  // two chains per row so that consecutive fmas do not wait on each other
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-              const f32x4 x = xp[jj * nchunk];
-              const uint32_t word = w[r][j][jj];
-              e = __builtin_fmaf((float)(word & 0xffu), x[0], e);
-              o = __builtin_fmaf((float)((word >> 8) & 0xffu), x[1], o);
-              e = __builtin_fmaf((float)((word >> 16) & 0xffu), x[2], e);
-              o = __builtin_fmaf((float)(word >> 24), x[3], o);
-            }
-            acc[r] += e + o;
+          for (int jj = 0; jj < 4; jj++) {
+            const f32x4 x = xp[jj * kPadChunks];
+            const uint32_t word = w[r][j][jj];
+            e = __builtin_fmaf((float)(word & 0xffu), x[0], e);
+            o = __builtin_fmaf((float)((word >> 8) & 0xffu), x[1], o);
+            e = __builtin_fmaf((float)((word >> 16) & 0xffu), x[2], e);
+            o = __builtin_fmaf((float)(word >> 24), x[3], o);
           }
+          acc[r] += e + o;
         }
       }
     }
   }
 };
+
+// Bytes of LDS one staged vector takes for a given tiling (padding included).
+__host__ __device__ constexpr size_t staged_bytes(int nch, bool u8) { return (size_t)nch * kWave * (u8 ? 64 : 16); }
+
+// Zero the padding chunks [nchunk, padchunks) of a staged vector.
+template <bool U8>
+__device__ __forceinline__ void zero_pad(void* vec, int nchunk, int padchunks) {
+  for (int c = nchunk + (int)threadIdx.x; c < padchunks; c += kThreads) {
+    if constexpr (!U8) {
+      reinterpret_cast<h8*>(vec)[c] = h8{};
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) reinterpret_cast<f32x4*>(vec)[jj * padchunks + c] = f32x4{};
+    }
+  }
+}
 
 // ---------------------------------------------------------------------------
 // uint8 matrices in the row-streaming kernels.  With w^[n][k] = q c_n ry_k + mx_n + my_k
@@ -187,14 +241,14 @@ struct RowBatch {
 // matrix-matrix kernel apply); the difference is below the rounding of the binary16 output.
 //
 // xr is staged "split": a lane's chunk c covers 16 codes = four 16-byte groups of xr, and
-// group j of chunk c lives at f32x4 index j * nchunk + c, so that consecutive lanes read
+// group j of chunk c lives at f32x4 index j * padchunks + c, so that consecutive lanes read
 // consecutive 16-byte LDS words.
 // ---------------------------------------------------------------------------
 constexpr int kQSums = 2;  // Sx, Smy
 
 // Thread-owned group g = 8 consecutive elements of the vector.
-__device__ __forceinline__ void stage_q(float* dst, int g, int K, h8 x, h8 ry, h8 my, float* part) {
-  const int nchunk = K >> 4;
+__device__ __forceinline__ void stage_q(float* dst, int g, int padchunks, h8 x, h8 ry, h8 my, float* part) {
+  const int nchunk = padchunks;
   f32x4 lo, hi;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -258,10 +312,11 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   const int C = a.C;
   const int nchunk = U8 ? (C >> 4) : (C >> 3);
   // binary16: the three mixed vectors; uint8: the three pre-scaled fp32 vectors xr (see stage_q)
-  constexpr int kElem = U8 ? 4 : 2;
+  constexpr int kPad = NCH * kWave;
+  constexpr size_t kVecBytes = staged_bytes(NCH, U8);
   unsigned char* kx = smem;
-  unsigned char* vx = kx + (size_t)kElem * C;
-  unsigned char* rx = vx + (size_t)kElem * C;
+  unsigned char* vx = kx + kVecBytes;
+  unsigned char* rx = vx + kVecBytes;
   __shared__ float qred[kWaves][kMaxSeg * kQSums];
 
   const int lane = threadIdx.x & (kWave - 1);
@@ -301,9 +356,9 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
     const h8 mv = mix8(ln.xx, sx, mixv);
     const h8 mr = mix8(ln.xx, sx, mixr);
     if constexpr (U8) {
-      stage_q(reinterpret_cast<float*>(kx), threadIdx.x, C, mk, qry[0], qmy[0], part + 0 * kQSums);
-      stage_q(reinterpret_cast<float*>(vx), threadIdx.x, C, mv, qry[1], qmy[1], part + 1 * kQSums);
-      stage_q(reinterpret_cast<float*>(rx), threadIdx.x, C, mr, qry[2], qmy[2], part + 2 * kQSums);
+      stage_q(reinterpret_cast<float*>(kx), threadIdx.x, kPad, mk, qry[0], qmy[0], part + 0 * kQSums);
+      stage_q(reinterpret_cast<float*>(vx), threadIdx.x, kPad, mv, qry[1], qmy[1], part + 1 * kQSums);
+      stage_q(reinterpret_cast<float*>(rx), threadIdx.x, kPad, mr, qry[2], qmy[2], part + 2 * kQSums);
     } else {
       reinterpret_cast<h8*>(kx)[threadIdx.x] = mk;
       reinterpret_cast<h8*>(vx)[threadIdx.x] = mv;
@@ -311,6 +366,9 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
     }
     if (blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
   }
+  zero_pad<U8>(kx, nchunk, kPad);
+  zero_pad<U8>(vx, nchunk, kPad);
+  zero_pad<U8>(rx, nchunk, kPad);
   if constexpr (U8) publish_qsums(part, 3 * kQSums, qred);
   __syncthreads();
   float qt[3 * kQSums];
@@ -329,7 +387,7 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       nxt.load(rows, nchunk, lane);
     }
     float acc[3];
-    cur.dot(xv, nchunk, lane, acc);
+    cur.dot(xv, lane, acc);
     float k = wave_sum(acc[0]);
     float v = wave_sum(acc[1]);
     float rr = wave_sum(acc[2]);
@@ -443,8 +501,9 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   const int nchunk = U8 ? (K >> 4) : (K >> 3);
   const size_t row_bytes = U8 ? (size_t)K : 2 * (size_t)K;
   // binary16: nvec staged activation vectors; uint8: one pre-scaled fp32 vector xr per segment
-  h1* vecs = reinterpret_cast<h1*>(smem);
-  float* qvecs = reinterpret_cast<float*>(smem);
+  constexpr int kPad = NCH * kWave;
+  constexpr size_t kVecBytes = staged_bytes(NCH, U8);
+  auto vec_at = [&](int i) { return smem + (size_t)i * kVecBytes; };
   __shared__ float qred[kWaves][kMaxSeg * kQSums];
   float qtv = 0.f;  // uint8: lane v holds total v of (Sx, Smy) x segments
 
@@ -479,13 +538,16 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     const void* xv[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      if constexpr (U8)
-        xv[r] = qvecs + (size_t)m.seg[r] * K;
-      else
-        xv[r] = vecs + (size_t)a.seg[m.seg[r]].vec * K;
+      xv[r] = vec_at(U8 ? m.seg[r] : a.seg[m.seg[r]].vec);
     }
     float acc[R];
-    b.dot(xv, nchunk, lane, acc);
+    bool same = true;
+#pragma unroll
+    for (int r = 1; r < R; r++) same = same && xv[r] == xv[0];
+    if (same)
+      b.dot_shared(xv[0], lane, acc);  // the usual case: a batch within one matrix
+    else
+      b.dot(xv, lane, acc);
     float mine = 0.f;
     int my_seg = 0, my_loc = 0;
 #pragma unroll
@@ -542,15 +604,32 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     for (int i = 0; i < kMaxSeg * kQSums; i++) part[i] = 0.f;
     if (a.prologue == P_COPY) {
       if constexpr (!U8) {
-        stage_vec<false>(vecs, a.vec0, K);
+        stage_vec<false>(reinterpret_cast<h1*>(vec_at(0)), a.vec0, K);
       } else {
-        for (int g = threadIdx.x; g < (K >> 3); g += kThreads) {
-          const h8 x = reinterpret_cast<const h8*>(a.vec0)[g];
+        // two groups per thread and pass, every load of a pass requested before its first use
+        const int ngrp = K >> 3;
+        for (int g = threadIdx.x; g < ngrp; g += 2 * kThreads) {
+          const int g2 = g + kThreads;
+          const bool two = g2 < ngrp;
+          h8 x[2], ry[2][kMaxSeg], my[2][kMaxSeg];
+          x[0] = reinterpret_cast<const h8*>(a.vec0)[g];
+          if (two) x[1] = reinterpret_cast<const h8*>(a.vec0)[g2];
 #pragma unroll
           for (int i = 0; i < kMaxSeg; i++)
-            if (i < a.nseg)
-              stage_q(qvecs + (size_t)i * K, g, K, x, *reinterpret_cast<const h8*>(a.seg[i].w.ry + 8 * g),
-                      *reinterpret_cast<const h8*>(a.seg[i].w.my + 8 * g), part + i * kQSums);
+            if (i < a.nseg) {
+              ry[0][i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + 8 * g);
+              my[0][i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + 8 * g);
+              if (two) {
+                ry[1][i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + 8 * g2);
+                my[1][i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + 8 * g2);
+              }
+            }
+#pragma unroll
+          for (int i = 0; i < kMaxSeg; i++)
+            if (i < a.nseg) {
+              stage_q(reinterpret_cast<float*>(vec_at(i)), g, kPad, x[0], ry[0][i], my[0][i], part + i * kQSums);
+              if (two) stage_q(reinterpret_cast<float*>(vec_at(i)), g2, kPad, x[1], ry[1][i], my[1][i], part + i * kQSums);
+            }
         }
       }
     } else {
@@ -558,11 +637,11 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       if (ln.active) {
         if constexpr (!U8) {
           if (a.prologue == P_LN) {
-            reinterpret_cast<h8*>(vecs)[threadIdx.x] = ln.xx;
+            reinterpret_cast<h8*>(vec_at(0))[threadIdx.x] = ln.xx;
           } else {
 #pragma unroll
             for (int i = 0; i < kMaxSeg; i++)
-              if (i < a.nvec) reinterpret_cast<h8*>(vecs + (size_t)i * K)[threadIdx.x] = mix8(ln.xx, sx, mixv[i]);
+              if (i < a.nvec) reinterpret_cast<h8*>(vec_at(i))[threadIdx.x] = mix8(ln.xx, sx, mixv[i]);
           }
         } else {
 #pragma unroll
@@ -577,13 +656,14 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
                   if (a.seg[i].vec == j) mx8 = mixv[j];
                 x = mix8(ln.xx, sx, mx8);
               }
-              stage_q(qvecs + (size_t)i * K, threadIdx.x, K, x, qry[i], qmy[i], part + i * kQSums);
+              stage_q(reinterpret_cast<float*>(vec_at(i)), threadIdx.x, kPad, x, qry[i], qmy[i], part + i * kQSums);
             }
           }
         }
         if (a.prologue == P_LN_MIX && blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
       }
     }
+    for (int i = 0; i < (U8 ? a.nseg : a.nvec); i++) zero_pad<U8>(vec_at(i), nchunk, kPad);
     if constexpr (U8) publish_qsums(part, a.nseg * kQSums, qred);
     __syncthreads();
     if constexpr (U8) qtv = gather_qsums(a.nseg * kQSums, qred);
@@ -592,17 +672,28 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   if constexpr (!MULTI) {
     if (g0 < g1) consume(A, mA, g0);  // the host guarantees g1 - g0 <= R
   } else {
+    // Two register sets alternate.  Each "fetch the next, consume the current" pair is straight-line
+    // code, so the loads of the next batch stay in flight while the current one is consumed.
     RowBatch<R, NCH, U8> B;
     Meta mB;
     int g = g0;
-    while (g < g1) {
-      if (g + R < g1) fetch(B, mB, g + R);
-      consume(A, mA, g);
-      g += R;
-      if (g >= g1) break;
-      if (g + R < g1) fetch(A, mA, g + R);
-      consume(B, mB, g);
-      g += R;
+    if (g < g1) {
+      for (;;) {
+        if (g + R >= g1) {
+          consume(A, mA, g);
+          break;
+        }
+        fetch(B, mB, g + R);
+        consume(A, mA, g);
+        g += R;
+        if (g + R >= g1) {
+          consume(B, mB, g);
+          break;
+        }
+        fetch(A, mA, g + R);
+        consume(B, mB, g);
+        g += R;
+      }
     }
   }
 }
@@ -758,6 +849,8 @@ static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
   *multi = true;
   int r = (kMaxLoads / 2) / nch;
   if (r < 1) r = 1;
+  // uint8 rows are half as long in bytes: eight of them per batch keep as many bytes in flight
+  if (u8 && r >= 8) return 8;
   if (r > 4) r = 4;
   return r;
 }
@@ -766,7 +859,7 @@ static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
 template <int R, int NCH>
 static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
   if (!multi) {
-    if constexpr (R * NCH <= kMaxLoads || R == 1) {
+    if constexpr ((R * NCH <= kMaxLoads && R <= 6) || R == 1) {
       if (u8)
         hipLaunchKernelGGL((rows_kernel<R, NCH, true, false>), dim3(grid), dim3(kThreads), lds, st, a);
       else
@@ -779,6 +872,10 @@ static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_
         hipLaunchKernelGGL((rows_kernel<R, NCH, true, true>), dim3(grid), dim3(kThreads), lds, st, a);
       else
         hipLaunchKernelGGL((rows_kernel<R, NCH, false, true>), dim3(grid), dim3(kThreads), lds, st, a);
+      return true;
+    } else if constexpr (R == 8 && NCH <= 2) {
+      if (!u8) return false;
+      hipLaunchKernelGGL((rows_kernel<R, NCH, true, true>), dim3(grid), dim3(kThreads), lds, st, a);
       return true;
     }
   }
@@ -794,6 +891,7 @@ static bool launch_rows_n(int R, bool u8, bool multi, int grid, size_t lds, hipS
     case 4: return launch_rows_rn<4, NCH>(u8, multi, grid, lds, st, a);
     case 5: return launch_rows_rn<5, NCH>(u8, multi, grid, lds, st, a);
     case 6: return launch_rows_rn<6, NCH>(u8, multi, grid, lds, st, a);
+    case 8: return launch_rows_rn<8, NCH>(u8, multi, grid, lds, st, a);
     default: return false;
   }
 }
@@ -804,7 +902,7 @@ static int launch_rows(const RowsArgs& a, bool u8, hipStream_t st, const char* w
   const int grid = decode_grid();
   bool multi = false;
   const int R = pick_r(a, grid, nch, u8, &multi);
-  const size_t lds = u8 ? 4 * (size_t)a.K * a.nseg : 2 * (size_t)a.K * a.nvec;
+  const size_t lds = staged_bytes(nch, u8) * (u8 ? a.nseg : a.nvec);
   FR_TRY(check_lds(lds));
   bool ok = false;
   switch (nch) {
@@ -920,9 +1018,10 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   a.xx_out = (h1*)xx_out; a.rwkv_out = w.rwkv;
   a.aa_out = aa_out; a.bb_out = bb_out; a.pp_out = pp_out;
   const bool u8 = kw->dtype == FRHIP_U8;
-  const size_t lds = (u8 ? 4 : 2) * (size_t)C * 3;
-  FR_TRY(check_lds(lds));
   const int nch = chunks_per_lane(C, u8);  // C <= 4096: at most 8 (fp16) or 4 (uint8)
+  const int nch_t = nch <= 1 ? 1 : nch == 2 ? 2 : nch <= 4 ? 4 : nch == 5 ? 5 : 8;  // compiled tilings
+  const size_t lds = staged_bytes(nch_t, u8) * 3;
+  FR_TRY(check_lds(lds));
 #define FR_ATT_FRONT(N)                                                                                   \
   do {                                                                                                    \
     if (u8)                                                                                               \

@@ -77,9 +77,18 @@ __device__ __forceinline__ float block_sum1(float v, float* red) {
 // kernels/cuda/att.cu:106-107: h(h(xx*m) + h(sx*h(1-m)))
 __device__ __forceinline__ h1 mix1(h1 xx, h1 sx, h1 m) { return (xx * m) + (sx * ((h1)1.0f - m)); }
 
-// kernels/cuda/att.cu:154-159: evaluated in double, narrowed to float, then to half
+// kernels/cuda/att.cu:154-159: evaluated in double, narrowed to float, then to half.
+// The double evaluation costs hundreds of cycles at the tail of a wave, so the value is first
+// formed in fp32 (a few units in the last place of error); only when that lies so close to the
+// midpoint of two binary16 values that the error could change the rounding, or in the binary16
+// subnormal range, is the double path taken.  The result is the double path's bit for bit.
 __device__ __forceinline__ h1 sigmoid_h(h1 x) {
-  double s = 1.0 / (1.0 + exp(-(double)(float)x));
+  const float xf = (float)x;
+  const float s32 = 1.0f / (1.0f + expf(-xf));
+  const uint32_t frac = __float_as_uint(s32) & 0x1FFFu;  // the 13 fp32 mantissa bits binary16 drops
+  const bool safe = s32 > 1e-4f && (frac < 0x1000u - 64u || frac > 0x1000u + 64u);
+  if (safe) return (h1)s32;
+  double s = 1.0 / (1.0 + exp(-(double)xf));
   return (h1)(float)s;
 }
 
