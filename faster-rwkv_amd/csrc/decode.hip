@@ -320,7 +320,8 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   __shared__ float qred[kWaves][kMaxSeg * kQSums];
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int gw = blockIdx.x * kWaves + threadIdx.x / kWave;
+  // wave-uniform, and known to the compiler as such: row addresses stay in scalar registers
+  const int gw = blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   int c0, c1;
   split_even(C, gridDim.x * kWaves, gw, c0, c1);
   const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
@@ -511,7 +512,10 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // The concatenated row space of all segments is split evenly over the waves of the grid;
   // global row g belongs to the segment s with start[s] <= g < start[s+1].
   int g0, g1;
-  split_even(a.start[a.nseg], gridDim.x * kWaves, blockIdx.x * kWaves + threadIdx.x / kWave, g0, g1);
+  // The wave index is made visibly uniform: otherwise the per-row lookups in the kernel arguments
+  // (segment table, row addresses) become vector loads that every weight load has to wait for.
+  split_even(a.start[a.nseg], gridDim.x * kWaves,
+             blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), g0, g1);
 
   struct Meta {
     int seg[R], loc[R];
