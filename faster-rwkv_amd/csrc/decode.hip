@@ -114,10 +114,15 @@ __device__ __forceinline__ h8 mix8(h8 xx, h8 sx, h8 m) {
   return o;
 }
 
-// Even split of `total` items over `parts`: part i gets [lo, hi).
-__device__ __forceinline__ void split_even(int total, int parts, int i, int& lo, int& hi) {
-  lo = (int)(((long long)total * i) / parts);
-  hi = (int)(((long long)total * (i + 1)) / parts);
+// Even split of items over the waves of the grid with the division done on the host:
+// wave i gets `base` items, the first `rem` waves one more.
+struct Split {
+  int base, rem;
+};
+
+__device__ __forceinline__ void split_even(Split sp, int i, int& lo, int& hi) {
+  lo = i * sp.base + (i < sp.rem ? i : sp.rem);
+  hi = lo + sp.base + (i < sp.rem ? 1 : 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -298,6 +303,7 @@ __device__ __forceinline__ float finish_q(float d, float rx, float mx, float sx,
 // ===========================================================================
 struct AttFrontV4 {
   int C;
+  Split split;  // channels over the waves of the grid
   const h1 *x, *sx, *ln_w, *ln_b, *mk, *mv, *mr;
   const float *aa, *bb, *pp, *td, *tf;
   WMat kw, vw, rw;
@@ -323,7 +329,7 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   // wave-uniform, and known to the compiler as such: row addresses stay in scalar registers
   const int gw = blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   int c0, c1;
-  split_even(C, gridDim.x * kWaves, gw, c0, c1);
+  split_even(a.split, gw, c0, c1);
   const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
 
   RowBatch<3, NCH, U8> cur;
@@ -454,6 +460,7 @@ struct Seg {
 
 struct RowsArgs {
   int K;          // length of every staged vector == K of every segment
+  Split split;    // rows of all segments over the waves of the grid (set at launch)
   int nseg, nvec; // segments, staged vectors
   int prologue;
   int start[kMaxSeg + 1];  // first global row of each segment; start[nseg] = total rows
@@ -514,25 +521,43 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   int g0, g1;
   // The wave index is made visibly uniform: otherwise the per-row lookups in the kernel arguments
   // (segment table, row addresses) become vector loads that every weight load has to wait for.
-  split_even(a.start[a.nseg], gridDim.x * kWaves,
-             blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), g0, g1);
+  split_even(a.split, blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), g0, g1);
 
   struct Meta {
     int seg[R], loc[R];
     h1 ex, er;  // epilogue operands of the row this lane finishes (lane < R)
   };
   // locate the rows of the batch starting at global row g and issue their loads
+  auto seg_of = [&](int gg) {
+    int sg = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxSeg; i++) sg += (i < a.nseg && gg >= a.start[i]) ? 1 : 0;
+    return sg;
+  };
   auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int g) {
     const void* rows[R];
+    const int glast = g + R - 1 < g1 ? g + R - 1 : g1 - 1;  // surplus slots re-read the last row
+    const int sg0 = seg_of(g);
+    if (sg0 == seg_of(glast)) {
+      // the usual case, a batch within one matrix: one lookup in the segment table
+      const int loc0 = g - a.start[sg0];
+      const unsigned char* base = a.seg[sg0].w.data;
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      const int gg = g + r < g1 ? g + r : g1 - 1;  // surplus slots re-read the last row
-      int sg = 0;
+      for (int r = 0; r < R; r++) {
+        const int gg = g + r < g1 ? g + r : g1 - 1;
+        m.seg[r] = sg0;
+        m.loc[r] = loc0 + (gg - g);
+        rows[r] = base + (size_t)m.loc[r] * row_bytes;
+      }
+    } else {
 #pragma unroll
-      for (int i = 1; i < kMaxSeg; i++) sg += (i < a.nseg && gg >= a.start[i]) ? 1 : 0;
-      m.seg[r] = sg;
-      m.loc[r] = gg - a.start[sg];
-      rows[r] = a.seg[sg].w.data + (size_t)m.loc[r] * row_bytes;
+      for (int r = 0; r < R; r++) {
+        const int gg = g + r < g1 ? g + r : g1 - 1;
+        const int sg = seg_of(gg);
+        m.seg[r] = sg;
+        m.loc[r] = gg - a.start[sg];
+        rows[r] = a.seg[sg].w.data + (size_t)m.loc[r] * row_bytes;
+      }
     }
     b.load(rows, nchunk, lane);
     m.ex = (h1)0.0f;
@@ -900,10 +925,17 @@ static bool launch_rows_n(int R, bool u8, bool multi, int grid, size_t lds, hipS
   }
 }
 
-static int launch_rows(const RowsArgs& a, bool u8, hipStream_t st, const char* what) {
-  const int nch = round_nch(chunks_per_lane(a.K, u8));
+static Split make_split(int total, int grid) {
+  const int waves = grid * kWaves;
+  return Split{total / waves, total % waves};
+}
+
+static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char* what) {
+  const int nch = round_nch(chunks_per_lane(args.K, u8));
   if (nch < 0) return set_error(FRHIP_ESHAPE, "K is too large for the row-streaming kernel (max 9216 fp16 / 18432 uint8)");
   const int grid = decode_grid();
+  RowsArgs a = args;
+  a.split = make_split(a.start[a.nseg], grid);
   bool multi = false;
   const int R = pick_r(a, grid, nch, u8, &multi);
   const size_t lds = staged_bytes(nch, u8) * (u8 ? a.nseg : a.nvec);
@@ -1015,6 +1047,7 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
 
   AttFrontV4 a;
   a.C = C;
+  a.split = make_split(C, grid);
   a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
   a.mk = (const h1*)k_mix; a.mv = (const h1*)v_mix; a.mr = (const h1*)r_mix;
   a.aa = aa; a.bb = bb; a.pp = pp; a.td = t_decay; a.tf = t_first;
