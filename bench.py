@@ -264,6 +264,10 @@ def main():
     kernel_ms, n_launch = measure_kernels(fr, cfg)
     abytes = algorithmic_bytes_per_token(cfg["wbytes"])
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
+    # HBM bytes per launch (average over the launches of one token) from the FETCH_SIZE / WRITE_SIZE
+    # hardware counters, scaled by a copy kernel of known size: measured with rocprofv3 --pmc on this
+    # command and kept in profiles/decode_rwkv4_1b5_fp16_hbm_traffic.md; not measured for uint8.
+    traffic = round((2916.6e6 + 2.2e6) / n_launch) if args.dtype == "fp16" else None
     out = {
         "metric": "decode tok/s (RWKV-4 1.5B-shaped, bs1, greedy)", "value": round(tok_s, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -273,7 +277,7 @@ def main():
         "config": {"workload": cfg["workload"], "strategy": cfg["strategy"], "steps": args.steps,
                    "host_loop": "Model::Run + D2H logits + host argmax per token"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "row-streaming matrix-vector kernels (att_front/att_out/ffn_front/ffn_out/head), "
                                "%d launches per token" % n_launch,
                      "bytes_per_token": abytes, "kernel_ms_per_token": round(kernel_ms, 4),
