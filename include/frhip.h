@@ -93,9 +93,11 @@ int frhip_graph_destroy(frhip_graph g);
 /* src: the reference's [K][N] row-major matrix on the device; dst: [N][K].
  * elem_bytes 1 (uint8 codes) or 2 (binary16). */
 int frhip_pack_transpose(const void *src_kn, void *dst_nk, int K, int N, int elem_bytes, frhip_stream s);
-/* Dequantise a packed uint8 weight into packed binary16, dst [N][K].  Every
- * operation in binary16, round-to-nearest-even:
- *   c = rx[n] / 255;  a = c * ry[k];  b = mx[n] + my[k];  w^ = fma(q, a, b). */
+/* Dequantise a packed uint8 weight into packed binary16, dst [N][K].  Evaluated in
+ * IEEE binary32 with one final round-to-nearest-even to binary16:
+ *   c = rx[n] / 255;  a = c * ry[k];  b = mx[n] + my[k];  w^ = h(fmaf(q, a, b)).
+ * frhip_gemm multiplies by exactly this w^; the one-token operators (frhip_gemv, att, ffn,
+ * head) evaluate the same formula in fp32 without the final rounding of w^. */
 int frhip_dequant_u8(const frhip_weight *w, void *dst_nk_f16, frhip_stream s);
 
 /* ---- primitive operators (names of kernels/kernels.h) ------------------------ */
