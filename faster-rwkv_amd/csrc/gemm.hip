@@ -131,54 +131,82 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
     store_tiles(k0);
     __syncthreads();
     if (k0 + BK < K) load_tiles(k0 + BK);
+    // all fragments of the K step are requested from LDS first; the MFMAs then start as the
+    // first ones arrive instead of paying the LDS latency once per 16-deep sub-step
+    h8 fa[BK / 16][MI], fb[BK / 16][2];
 #pragma unroll
-    for (int ks = 0; ks < BK; ks += 16) {
-      h8 fa[MI], fb[2];
-      const int kofs = ks + (lane >> 5) * 8;
+    for (int kq = 0; kq < BK / 16; kq++) {
+      const int kofs = kq * 16 + (lane >> 5) * 8;
 #pragma unroll
-      for (int i = 0; i < MI; i++) fa[i] = *reinterpret_cast<const h8*>(&As[wm * (BM / 2) + i * 32 + (lane & 31)][kofs]);
+      for (int i = 0; i < MI; i++)
+        fa[kq][i] = *reinterpret_cast<const h8*>(&As[wm * (BM / 2) + i * 32 + (lane & 31)][kofs]);
 #pragma unroll
-      for (int j = 0; j < 2; j++) fb[j] = *reinterpret_cast<const h8*>(&Bs[wn * 64 + j * 32 + (lane & 31)][kofs]);
+      for (int j = 0; j < 2; j++) fb[kq][j] = *reinterpret_cast<const h8*>(&Bs[wn * 64 + j * 32 + (lane & 31)][kofs]);
+    }
+#pragma unroll
+    for (int kq = 0; kq < BK / 16; kq++)
 #pragma unroll
       for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kq][i], fb[kq][j], acc[i][j], 0, 0, 0);
   }
 
-  // epilogue: acc[i][j][v] is C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the 32x32 tile
+  // epilogue: acc[i][j][v] is C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the 32x32 tile.
+  // The epilogue kind is uniform over the launch segment: branch once, and for the kinds that read
+  // operands request all 16 of a tile before the first is used.
+  auto for_tile = [&](int i, int j, auto&& f) {
+    const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+      f(v, row < M && col < N, (size_t)(row < M ? row : M - 1) * N + (col < N ? col : N - 1));
+    }
+  };
 #pragma unroll
   for (int i = 0; i < MI; i++) {
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (row < M && col < N) {
-          const float s = acc[i][j][v];
-          const size_t o = (size_t)row * N + col;
-          switch (sg.epi) {
-            case G_STORE_F16: static_cast<h1*>(sg.out)[o] = (h1)s; break;
-            case G_STORE_F32: static_cast<float*>(sg.out)[o] = s; break;
-            case G_SIGMOID: static_cast<h1*>(sg.out)[o] = sigmoid_h((h1)s); break;
-            case G_RELU2: {
-              const h1 t = (h1)s;
-              static_cast<h1*>(sg.out)[o] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
-              break;
-            }
-            case G_SILU: static_cast<h1*>(sg.out)[o] = silu_h((h1)s); break;
-            case G_RESIDUAL: static_cast<h1*>(sg.out)[o] = a.res_x[o] + (h1)s; break;
-            case G_FFN_OUT: {
-              h1 r = __builtin_fmaf16((h1)s, a.res_r[o], a.res_x[o]);
-              if (a.div2) r = r / (h1)2.0f;
-              static_cast<h1*>(sg.out)[o] = r;
-              break;
-            }
-            default: break;
-          }
+      const f16v& c = acc[i][j];
+      switch (sg.epi) {
+        case G_STORE_F16:
+          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = (h1)c[v]; });
+          break;
+        case G_STORE_F32:
+          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<float*>(sg.out)[o] = c[v]; });
+          break;
+        case G_SIGMOID:
+          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = sigmoid_h((h1)c[v]); });
+          break;
+        case G_RELU2:
+          for_tile(i, j, [&](int v, bool ok, size_t o) {
+            const h1 t = (h1)c[v];
+            if (ok) static_cast<h1*>(sg.out)[o] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
+          });
+          break;
+        case G_SILU:
+          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = silu_h((h1)c[v]); });
+          break;
+        case G_RESIDUAL: {
+          h1 rx[16];
+          for_tile(i, j, [&](int v, bool, size_t o) { rx[v] = a.res_x[o]; });
+          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = rx[v] + (h1)c[v]; });
+          break;
         }
+        case G_FFN_OUT: {
+          h1 rx[16], rr[16];
+          for_tile(i, j, [&](int v, bool, size_t o) {
+            rx[v] = a.res_x[o];
+            rr[v] = a.res_r[o];
+          });
+          for_tile(i, j, [&](int v, bool ok, size_t o) {
+            h1 r = __builtin_fmaf16((h1)c[v], rr[v], rx[v]);
+            if (a.div2) r = r / (h1)2.0f;
+            if (ok) static_cast<h1*>(sg.out)[o] = r;
+          });
+          break;
+        }
+        default: break;
       }
     }
   }

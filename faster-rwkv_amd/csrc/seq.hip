@@ -73,6 +73,113 @@ __global__ __launch_bounds__(256) void ln_mix_seq_kernel(LnMixSeq a) {
   }
 }
 
+// The same for C % 8 == 0, C <= 8 * 256 * NG: a workgroup takes kLnRows consecutive rows plus the
+// row before them (the token shift of its first row), every thread owns NG groups of 8 elements
+// of every row in registers, all rows are loaded up front and their statistics reduced together
+// (two barriers per workgroup), and the mixed rows leave as 16-byte stores.
+constexpr int kLnRows = 4;
+
+template <int NG>
+__global__ __launch_bounds__(256) void ln_mix_rows_kernel(LnMixSeq a) {
+  constexpr int NR = kLnRows + 1;  // row 0 is the row before the workgroup's first
+  __shared__ float red[2][4][NR];
+  const int C = a.C, ngrp = C >> 3;
+  const int t0 = blockIdx.x * kLnRows;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  h8 xr[NR][NG], gam[NG], bet[NG];
+  bool own[NG];
+#pragma unroll
+  for (int n = 0; n < NG; n++) {
+    const int g = threadIdx.x + n * 256;
+    own[n] = g < ngrp;
+    const int gc = own[n] ? g : 0;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      int t = t0 - 1 + r;
+      t = t < 0 ? 0 : (t < a.T ? t : a.T - 1);
+      xr[r][n] = reinterpret_cast<const h8*>(a.x + (size_t)t * C)[gc];
+    }
+    gam[n] = reinterpret_cast<const h8*>(a.ln_w)[gc];
+    bet[n] = reinterpret_cast<const h8*>(a.ln_b)[gc];
+  }
+  h8 shift0[NG];  // the shift state, used instead of LN(row -1) by the first workgroup
+  if (t0 == 0) {
+#pragma unroll
+    for (int n = 0; n < NG; n++) shift0[n] = reinterpret_cast<const h8*>(a.state)[own[n] ? threadIdx.x + n * 256 : 0];
+  }
+  float mean[NR], inv[NR];
+  {
+    float s[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      s[r] = 0.f;
+#pragma unroll
+      for (int n = 0; n < NG; n++)
+        if (own[n])
+#pragma unroll
+          for (int i = 0; i < 8; i++) s[r] += (float)xr[r][n][i];
+      s[r] = wave_sum(s[r]);
+      if (lane == 0) red[0][wv][r] = s[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NR; r++) mean[r] = (((red[0][0][r] + red[0][1][r]) + red[0][2][r]) + red[0][3][r]) / (float)C;
+    float q[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      q[r] = 0.f;
+#pragma unroll
+      for (int n = 0; n < NG; n++)
+        if (own[n])
+#pragma unroll
+          for (int i = 0; i < 8; i++) {
+            const float d = (float)xr[r][n][i] - mean[r];
+            q[r] += d * d;
+          }
+      q[r] = wave_sum(q[r]);
+      if (lane == 0) red[1][wv][r] = q[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      float var = (((red[1][0][r] + red[1][1][r]) + red[1][2][r]) + red[1][3][r]) / (float)C;
+      var = var > 0.f ? var : 0.f;
+      inv[r] = 1.0f / sqrtf(var + 1e-5f);
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < NG; n++) {
+    if (!own[n]) continue;
+    const int g = threadIdx.x + n * 256;
+    h8 prev;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      h8 xx;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {  // kernels/cuda/layer_norm.cu:60-69: half, * gamma in half, + beta in half
+        const h1 nrm = (h1)(((float)xr[r][n][i] - mean[r]) * inv[r]);
+        xx[i] = (nrm * gam[n][i]) + bet[n][i];
+      }
+      if (r == 0) {
+        prev = t0 == 0 ? shift0[n] : xx;
+        continue;
+      }
+      const int t = t0 + r - 1;
+      if (t < a.T) {
+        for (int m = 0; m < a.nmix; m++) {
+          const h8 mx = reinterpret_cast<const h8*>(a.mix[m])[g];
+          h8 o;
+#pragma unroll
+          for (int i = 0; i < 8; i++) o[i] = mix1(xx[i], prev[i], mx[i]);
+          reinterpret_cast<h8*>(a.out[m] + (size_t)t * C)[g] = o;
+        }
+        if (t == a.T - 1) reinterpret_cast<h8*>(a.xx_last)[g] = xx;
+      }
+      prev = xx;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // RWKV-4 WKV scan.  k, v [T][C] fp32; r [T][C] half (already through the sigmoid),
 // overwritten with r * half(wkv).
@@ -108,25 +215,43 @@ __global__ __launch_bounds__(256) void wkv4_local_kernel(Wkv4Seq a) {
   a.lp[o] = pp;
 }
 
-__global__ __launch_bounds__(256) void wkv4_carry_kernel(Wkv4Seq a) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
+// The serial pass over the chunks.  A channel's step needs three values per chunk; they are read
+// eight chunks at a time ahead of the recurrence, so the pass costs one memory round trip per
+// eight chunks instead of one per chunk.
+__global__ __launch_bounds__(64) void wkv4_carry_kernel(Wkv4Seq a) {
+  const int c = blockIdx.x * 64 + threadIdx.x;
   if (c >= a.C) return;
+  constexpr int PF = 8;
   const float w = a.w[c];
   float aa = a.aa[c], bb = a.bb[c], pp = a.pp[c];
-  for (int ch = 0; ch < a.nchunk; ch++) {
-    const size_t o = (size_t)ch * a.C + c;
-    a.sa[o] = aa;
-    a.sb[o] = bb;
-    a.sp[o] = pp;
-    const int len = min(a.Lc, a.T - ch * a.Lc);
-    // the incoming state decays by len steps; the chunk's own tokens contribute its local state
-    const float pd = pp + (float)len * w;
-    const float lp = a.lp[o];
-    const float p = (pd > lp) ? pd : lp;
-    const float e1 = expf(pd - p), e2 = expf(lp - p);
-    aa = e1 * aa + e2 * a.la[o];
-    bb = e1 * bb + e2 * a.lb[o];
-    pp = p;
+  for (int ch0 = 0; ch0 < a.nchunk; ch0 += PF) {
+    float lp[PF], la[PF], lb[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int ch = ch0 + i < a.nchunk ? ch0 + i : a.nchunk - 1;
+      const size_t o = (size_t)ch * a.C + c;
+      lp[i] = a.lp[o];
+      la[i] = a.la[o];
+      lb[i] = a.lb[o];
+    }
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int ch = ch0 + i;
+      if (ch < a.nchunk) {
+        const size_t o = (size_t)ch * a.C + c;
+        a.sa[o] = aa;
+        a.sb[o] = bb;
+        a.sp[o] = pp;
+        const int len = min(a.Lc, a.T - ch * a.Lc);
+        // the incoming state decays by len steps; the chunk's own tokens contribute its local state
+        const float pd = pp + (float)len * w;
+        const float p = (pd > lp[i]) ? pd : lp[i];
+        const float e1 = expf(pd - p), e2 = expf(lp[i] - p);
+        aa = e1 * aa + e2 * la[i];
+        bb = e1 * bb + e2 * lb[i];
+        pp = p;
+      }
+    }
   }
 }
 
@@ -214,18 +339,30 @@ __global__ __launch_bounds__(256) void wkv5_local_kernel(Wkv5Seq a) {
   for (int ii = 0; ii < 16; ii++) dst[(ig * 16 + ii) * S5 + j] = s[ii];
 }
 
+// The serial pass over the chunks, one state element per thread; the chunks' local end states are
+// read eight at a time ahead of the recurrence.
 __global__ __launch_bounds__(256) void wkv5_carry_kernel(Wkv5Seq a) {
   const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;  // element of [H][64][64]
   const size_t per = (size_t)a.H * S5 * S5;
   if (e >= per) return;
+  constexpr int PF = 8;
   const int i = (int)((e / S5) % S5), h = (int)(e / (S5 * S5));
   const float w = a.w[a.uw_head ? h : h * S5 + i];
   float s = a.s[e];
-  for (int ch = 0; ch < a.nchunk; ch++) {
-    a.sin[(size_t)ch * per + e] = s;
-    const int len = min(a.Lc, a.T - ch * a.Lc);
-    for (int q = 0; q < len; q++) s = w * s;  // decay of the incoming state over the chunk
-    s = s + a.loc[(size_t)ch * per + e];
+  for (int ch0 = 0; ch0 < a.nchunk; ch0 += PF) {
+    float loc[PF];
+#pragma unroll
+    for (int j = 0; j < PF; j++) loc[j] = a.loc[(size_t)(ch0 + j < a.nchunk ? ch0 + j : a.nchunk - 1) * per + e];
+#pragma unroll
+    for (int j = 0; j < PF; j++) {
+      const int ch = ch0 + j;
+      if (ch < a.nchunk) {
+        a.sin[(size_t)ch * per + e] = s;
+        const int len = min(a.Lc, a.T - ch * a.Lc);
+        for (int q = 0; q < len; q++) s = w * s;  // decay of the incoming state over the chunk
+        s = s + loc[j];
+      }
+    }
   }
 }
 
@@ -321,7 +458,13 @@ static int launch_ln_mix(int T, int C, const void* x, const void* state, const v
     a.out[i] = out[i];
   }
   a.xx_last = (h1*)xx_last;
-  hipLaunchKernelGGL(ln_mix_seq_kernel, dim3(T), dim3(256), 4 * (size_t)C, st, a);
+  const int nwg = (T + kLnRows - 1) / kLnRows;
+  if (C % 8 == 0 && C <= 2048)
+    hipLaunchKernelGGL(ln_mix_rows_kernel<1>, dim3(nwg), dim3(256), 0, st, a);
+  else if (C % 8 == 0 && C <= 4096)
+    hipLaunchKernelGGL(ln_mix_rows_kernel<2>, dim3(nwg), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL(ln_mix_seq_kernel, dim3(T), dim3(256), 4 * (size_t)C, st, a);
   return check_launch("ln_mix_seq");
 }
 
@@ -453,7 +596,7 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   q.aa_out = aa_out; q.bb_out = bb_out; q.pp_out = pp_out;
   dim3 grid((C + 255) / 256, q.nchunk);
   hipLaunchKernelGGL(wkv4_local_kernel, grid, dim3(256), 0, st, q);
-  hipLaunchKernelGGL(wkv4_carry_kernel, dim3((C + 255) / 256), dim3(256), 0, st, q);
+  hipLaunchKernelGGL(wkv4_carry_kernel, dim3((C + 63) / 64), dim3(64), 0, st, q);
   hipLaunchKernelGGL(wkv4_apply_kernel, grid, dim3(256), 0, st, q);
   FR_TRY(check_launch("wkv4_seq"));
 
