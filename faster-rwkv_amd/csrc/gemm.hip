@@ -4,7 +4,8 @@
 //
 // Both operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
 // a lane's A (or B) fragment is 8 consecutive k of one row, i.e. one 16-byte load.
-// Workgroup tile 128x128 (64x128 for launches that would otherwise leave CUs idle), K step 64,
+// Workgroup tile 128x128 (64x128 for launches that would otherwise leave CUs idle), K step 64 (128 for
+// launches of about one workgroup per CU),
 // 256 threads = 2x2 waves of 64x64 (2x2 MFMA tiles, 64 fp32 accumulators per lane).  Tiles of X and Wt go global -> registers -> LDS
 // (rows padded by 16 bytes against bank conflicts); the loads of step k+1 are issued
 // before the MFMAs of step k.  uint8 weights are dequantised to binary16 on their way
@@ -24,16 +25,24 @@ namespace frhip {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int BN = 128, BK = 64, LDSK = BK + 8;
+constexpr int BN = 128;
 constexpr int kGemmThreads = 256;
 // BM = 128 (waves 2 x 2 of 64 x 64) or 64 (waves of 32 x 64), for launches that would otherwise
-// leave compute units idle.
-template <int BM, bool U8>
+// leave compute units idle.  BK = 64, or 128 for launches with about one workgroup per CU: with a
+// single wave per SIMD nothing hides the round trip of the next tile's loads, so a K step lasts
+// about one memory latency whatever its depth, and a deeper step halves their number.
+template <int BM, int BK, bool U8>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
-  constexpr int MI = BM / 64;   // 32-row MFMA blocks per wave
-  constexpr int AC = BM / 32;   // 16-byte chunks of the A tile per thread
-  __shared__ __attribute__((aligned(16))) h1 As[BM][LDSK];
-  __shared__ __attribute__((aligned(16))) h1 Bs[BN][LDSK];
+  constexpr int LDSK = BK + 8;
+  constexpr int MI = BM / 64;                      // 32-row MFMA blocks per wave
+  constexpr int CPR = BK / 8;                      // 16-byte chunks of 8 halves per tile row
+  constexpr int AC = BM * CPR / kGemmThreads;      // chunks of the A tile per thread
+  constexpr int BC = BN * CPR / kGemmThreads;      // chunks of a binary16 B tile per thread
+  constexpr int QPR = BK / 16;                     // 16-code chunks per tile row (uint8)
+  constexpr int QC = BN * QPR / kGemmThreads;      // chunks of a uint8 B tile per thread
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];  // gemm_lds_bytes(BM, BK)
+  h1* const As = reinterpret_cast<h1*>(gemm_smem);  // [BM][LDSK]
+  h1* const Bs = As + BM * LDSK;                    // [BN][LDSK]
 
   // which segment does this N-tile belong to
   int sidx = 0;
@@ -51,67 +60,69 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
   // global -> register staging: a tile is 128 rows x 64 k.
   //   A (binary16): 1024 chunks of 8 halves, 4 per thread: chunk c -> row c/8, k (c%8)*8
   //   B binary16: same.  B uint8: 512 chunks of 16 codes, 2 per thread: row c/4, k (c%4)*16
-  h8 ra[AC];
-  h8 rb[4];
-  u32x4 rq[2];
-  auto load_tiles = [&](int k0) {
+  struct Stage {
+    h8 ra[AC];
+    h8 rb[U8 ? 1 : BC];
+    u32x4 rq[U8 ? QC : 1];
+  };
+  auto load_tiles = [&](Stage& st, int k0) {
 #pragma unroll
     for (int i = 0; i < AC; i++) {
       const int c = tid + i * kGemmThreads;
-      int row = m0 + (c >> 3);
+      int row = m0 + c / CPR;
       row = row < M ? row : M - 1;  // rows past M are computed on a copy of the last row and never stored
-      ra[i] = *reinterpret_cast<const h8*>(sg.A + (size_t)row * K + k0 + (c & 7) * 8);
+      st.ra[i] = *reinterpret_cast<const h8*>(sg.A + (size_t)row * K + k0 + (c % CPR) * 8);
     }
     if constexpr (!U8) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
+      for (int i = 0; i < BC; i++) {
         const int c = tid + i * kGemmThreads;
-        int row = n0 + (c >> 3);
+        int row = n0 + c / CPR;
         row = row < N ? row : N - 1;
-        rb[i] = __builtin_nontemporal_load(reinterpret_cast<const h8*>(sg.B + ((size_t)row * K + k0 + (c & 7) * 8) * 2));
+        st.rb[i] = __builtin_nontemporal_load(reinterpret_cast<const h8*>(sg.B + ((size_t)row * K + k0 + (c % CPR) * 8) * 2));
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
+      for (int i = 0; i < QC; i++) {
         const int c = tid + i * kGemmThreads;
-        int row = n0 + (c >> 2);
+        int row = n0 + c / QPR;
         row = row < N ? row : N - 1;
-        rq[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sg.B + (size_t)row * K + k0 + (c & 3) * 16));
+        st.rq[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sg.B + (size_t)row * K + k0 + (c % QPR) * 16));
       }
     }
   };
-  auto store_tiles = [&](int k0) {
+  auto store_tiles = [&](const Stage& st, int k0) {
 #pragma unroll
     for (int i = 0; i < AC; i++) {
       const int c = tid + i * kGemmThreads;
-      *reinterpret_cast<h8*>(&As[c >> 3][(c & 7) * 8]) = ra[i];
+      *reinterpret_cast<h8*>(&As[(c / CPR) * LDSK + (c % CPR) * 8]) = st.ra[i];
     }
     if constexpr (!U8) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
+      for (int i = 0; i < BC; i++) {
         const int c = tid + i * kGemmThreads;
-        *reinterpret_cast<h8*>(&Bs[c >> 3][(c & 7) * 8]) = rb[i];
+        *reinterpret_cast<h8*>(&Bs[(c / CPR) * LDSK + (c % CPR) * 8]) = st.rb[i];
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
+      for (int i = 0; i < QC; i++) {
         const int c = tid + i * kGemmThreads;
-        int row = n0 + (c >> 2);
+        int row = n0 + c / QPR;
         row = row < N ? row : N - 1;
-        const int kk = k0 + (c & 3) * 16;
+        const int kk = k0 + (c % QPR) * 16;
         const float c2 = dequant_c(sg.rx[row]);
         const float m2 = (float)sg.mx[row];
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
           const h8 ry = *reinterpret_cast<const h8*>(sg.ry + kk + hh * 8);
           const h8 my = *reinterpret_cast<const h8*>(sg.my + kk + hh * 8);
-          const uint32_t w0 = rq[i][2 * hh], w1 = rq[i][2 * hh + 1];
+          const uint32_t w0 = st.rq[i][2 * hh], w1 = st.rq[i][2 * hh + 1];
           h2 p0 = dequant_pair<0>(w0, c2, m2, ry.s01, my.s01);
           h2 p1 = dequant_pair<1>(w0, c2, m2, ry.s23, my.s23);
           h2 p2 = dequant_pair<0>(w1, c2, m2, ry.s45, my.s45);
           h2 p3 = dequant_pair<1>(w1, c2, m2, ry.s67, my.s67);
           h8 o = {p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
-          *reinterpret_cast<h8*>(&Bs[c >> 2][(c & 3) * 16 + hh * 8]) = o;
+          *reinterpret_cast<h8*>(&Bs[(c / QPR) * LDSK + (c % QPR) * 16 + hh * 8]) = o;
         }
       }
     }
@@ -125,31 +136,41 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-  load_tiles(0);
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    __syncthreads();  // everyone is done reading the previous tile
-    store_tiles(k0);
-    __syncthreads();
-    if (k0 + BK < K) load_tiles(k0 + BK);
-    // all fragments of the K step are requested from LDS first; the MFMAs then start as the
-    // first ones arrive instead of paying the LDS latency once per 16-deep sub-step
-    h8 fa[BK / 16][MI], fb[BK / 16][2];
+  // the fragments of FG * 16 k are requested from LDS together; the MFMAs then start as the first
+  // ones arrive instead of paying the LDS latency once per 16-deep sub-step
+  auto compute_tile = [&]() {
+    constexpr int FG = 4;
 #pragma unroll
-    for (int kq = 0; kq < BK / 16; kq++) {
-      const int kofs = kq * 16 + (lane >> 5) * 8;
+    for (int kh = 0; kh < BK; kh += FG * 16) {
+      h8 fa[FG][MI], fb[FG][2];
 #pragma unroll
-      for (int i = 0; i < MI; i++)
-        fa[kq][i] = *reinterpret_cast<const h8*>(&As[wm * (BM / 2) + i * 32 + (lane & 31)][kofs]);
+      for (int kq = 0; kq < FG; kq++) {
+        const int kofs = kh + kq * 16 + (lane >> 5) * 8;
 #pragma unroll
-      for (int j = 0; j < 2; j++) fb[kq][j] = *reinterpret_cast<const h8*>(&Bs[wn * 64 + j * 32 + (lane & 31)][kofs]);
-    }
-#pragma unroll
-    for (int kq = 0; kq < BK / 16; kq++)
-#pragma unroll
-      for (int i = 0; i < MI; i++)
+        for (int i = 0; i < MI; i++)
+          fa[kq][i] = *reinterpret_cast<const h8*>(&As[(wm * (BM / 2) + i * 32 + (lane & 31)) * LDSK + kofs]);
 #pragma unroll
         for (int j = 0; j < 2; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kq][i], fb[kq][j], acc[i][j], 0, 0, 0);
+          fb[kq][j] = *reinterpret_cast<const h8*>(&Bs[(wn * 64 + j * 32 + (lane & 31)) * LDSK + kofs]);
+      }
+#pragma unroll
+      for (int kq = 0; kq < FG; kq++)
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kq][i], fb[kq][j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  Stage s0;
+  load_tiles(s0, 0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();  // everyone is done reading the previous tile
+    store_tiles(s0, k0);
+    __syncthreads();
+    if (k0 + BK < K) load_tiles(s0, k0 + BK);
+    compute_tile();
   }
 
   // epilogue: acc[i][j][v] is C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the 32x32 tile.
@@ -212,9 +233,38 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
   }
 }
 
+static constexpr size_t gemm_lds_bytes(int bm, int bk) { return (size_t)(bm + BN) * (bk + 8) * 2; }
+
+// Tiles above 64 KB of LDS need the limit raised once per kernel.
+template <int BM, int BK, bool U8>
+static void gemm_launch_one(dim3 grid, hipStream_t st, const GemmArgs& a) {
+  constexpr size_t lds = gemm_lds_bytes(BM, BK);
+  static bool raised = false;
+  if (lds > 64 * 1024 && !raised) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<BM, BK, U8>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL((gemm_kernel<BM, BK, U8>), grid, dim3(kGemmThreads), lds, st, a);
+}
+#define FR_GEMM_LAUNCH(BM_, BK_)                         \
+  do {                                                   \
+    if (u8)                                              \
+      gemm_launch_one<BM_, BK_, true>(grid, st, a);      \
+    else                                                 \
+      gemm_launch_one<BM_, BK_, false>(grid, st, a);     \
+  } while (0)
+
+// FRHIP_GEMM_BK=64|128 forces the K-step depth (measurement aid); default: 128 where K allows
+// (256 was measured no faster than 128).
+static int env_bk() {
+  const char* e = getenv("FRHIP_GEMM_BK");
+  return e ? atoi(e) : 0;
+}
+
 int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what) {
   if (a.M <= 0) return 0;
-  if (a.K <= 0 || a.K % BK != 0) return set_error(FRHIP_ESHAPE, "gemm: K must be a positive multiple of 64");
+  if (a.K <= 0 || a.K % 64 != 0) return set_error(FRHIP_ESHAPE, "gemm: K must be a positive multiple of 64");
   int tiles = 0;
   for (int s = 0; s < a.nseg; s++) {
     a.tile_start[s] = tiles;
@@ -224,18 +274,17 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what) {
   a.tile_start[a.nseg] = tiles;
   // 128-row tiles unless that leaves fewer than ~1.5 workgroups per CU; then 64-row tiles
   const int m128 = (a.M + 127) / 128;
-  if ((long)tiles * m128 < (long)compute_units() * 3 / 2) {
+  static const int force_bm = getenv("FRHIP_GEMM_BM") ? atoi(getenv("FRHIP_GEMM_BM")) : 0;  // measurement aid
+  const bool small = force_bm ? force_bm == 64 : (long)tiles * m128 < (long)compute_units() * 3 / 2;
+  static const int force_bk = env_bk();
+  const bool deep = force_bk ? force_bk == 128 : true;
+  const bool deep_ok = deep && a.K % 128 == 0;
+  if (small) {
     dim3 grid(tiles, (a.M + 63) / 64);
-    if (u8)
-      hipLaunchKernelGGL((gemm_kernel<64, true>), grid, dim3(kGemmThreads), 0, st, a);
-    else
-      hipLaunchKernelGGL((gemm_kernel<64, false>), grid, dim3(kGemmThreads), 0, st, a);
+    if (deep_ok) FR_GEMM_LAUNCH(64, 128); else FR_GEMM_LAUNCH(64, 64);
   } else {
     dim3 grid(tiles, m128);
-    if (u8)
-      hipLaunchKernelGGL((gemm_kernel<128, true>), grid, dim3(kGemmThreads), 0, st, a);
-    else
-      hipLaunchKernelGGL((gemm_kernel<128, false>), grid, dim3(kGemmThreads), 0, st, a);
+    if (deep_ok) FR_GEMM_LAUNCH(128, 128); else FR_GEMM_LAUNCH(128, 64);
   }
   return check_launch(what);
 }
