@@ -181,6 +181,26 @@ def prefill_extra(fr):
             "prefill_frac_of_2500_TFLOPs": round(flops / best / 2.5e15, 4)}
 
 
+def rwkv5_extra(fr):
+    """BASELINE configuration 5: RWKV-5.2 3B-shaped uint8 model, T=512 seq-mode prefill then 256
+    greedy one-token steps."""
+    m = fr.Model("synthetic:v=5.2,L=32,C=2560,F=8960,V=65536,H=40,seed=1238", "hip int8")
+    ids = np.random.default_rng(44).integers(0, V_, 512)
+    best = 1e9
+    for _ in range(3):
+        m.reset()
+        t0 = time.perf_counter()
+        lg = m.run(ids)
+        best = min(best, time.perf_counter() - t0)
+    m.greedy(int(np.argmax(lg)), 16)
+    _, secs = m.greedy(17, 256)
+    m.close()
+    wbytes = 32 * 85196800 + 167772160  # uint8 codes of every matrix, once per token
+    return {"rwkv5_3b_int8_prefill_T512_ms": round(best * 1e3, 2), "rwkv5_3b_int8_prefill_tok_s": round(512 / best, 1),
+            "rwkv5_3b_int8_decode_tok_s": round(256 / secs, 1),
+            "rwkv5_3b_int8_decode_weight_GBs": round(wbytes * 256 / secs / 1e9, 1)}
+
+
 def cpu_baseline(seconds_budget=20.0):
     """The oracle's fp32 one-token forward on the host cores (OpenMP over output columns), on
     the same architecture with the depth cut to 2 layers + head to bound the run; the
@@ -298,6 +318,7 @@ def main():
         extra[other + "_gemv_GBs"] = round(ob / (okms * 1e-3) / 1e9, 1)
         extra[other + "_gemv_frac_of_hbm_peak"] = round(ob / (okms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         extra.update(prefill_extra(fr))
+        extra.update(rwkv5_extra(fr))
         extra.update(probe_bandwidth(fr))
         out["extra"] = extra
     out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()

@@ -152,7 +152,9 @@ struct RowBatch {
     }
   }
 
-  // All rows against the same staged vector: each chunk of it is read from LDS once.
+  // All rows against one staged vector, each chunk of which is read from LDS once.  Binary16 rows:
+  // acc[r] = sum_k w[k] x[k] against a binary16 vector; uint8 rows: acc[r] = sum_k q[k] xr[k]
+  // against an fp32 vector staged by stage_q.
   __device__ __forceinline__ void dot_shared(const void* xv, int lane, float (&acc)[R]) const {
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
@@ -186,36 +188,6 @@ struct RowBatch {
     }
   }
 
-  // Binary16 rows: acc[r] = sum_k w[k] x[k] against a binary16 vector.  uint8 rows:
-  // acc[r] = sum_k q[k] xr[k] against an fp32 vector staged by stage_q.
-  __device__ __forceinline__ void dot(const void* const (&xv)[R], int lane, float (&acc)[R]) const {
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.f;
-#pragma unroll
-    for (int j = 0; j < NCH; j++) {
-      const int c = lane + j * kWave;
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        if constexpr (!U8) {
-          h8 x = reinterpret_cast<const h8*>(xv[r])[c];
-          acc[r] = dot8acc(w[r][j], x, acc[r]);
-        } else {
-          const f32x4* xp = reinterpret_cast<const f32x4*>(xv[r]) + c;
-          float e = 0.f, o = 0.f;  // two chains per row so that consecutive fmas do not wait on each other
-#pragma unroll
-          for (int jj = 0; jj < 4; jj++) {
-            const f32x4 x = xp[jj * kPadChunks];
-            const uint32_t word = w[r][j][jj];
-            e = __builtin_fmaf((float)(word & 0xffu), x[0], e);
-            o = __builtin_fmaf((float)((word >> 8) & 0xffu), x[1], o);
-            e = __builtin_fmaf((float)((word >> 16) & 0xffu), x[2], e);
-            o = __builtin_fmaf((float)(word >> 24), x[3], o);
-          }
-          acc[r] += e + o;
-        }
-      }
-    }
-  }
 };
 
 // Bytes of LDS one staged vector takes for a given tiling (padding included).
@@ -332,11 +304,22 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   split_even(a.split, gw, c0, c1);
   const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
 
-  RowBatch<3, NCH, U8> cur;
+  // the three rows of a channel as three one-row batches: each multiplies its own staged vector
+  struct Rows3 {
+    RowBatch<1, NCH, U8> k, v, r;
+  };
+  auto load3 = [&](Rows3& b, int n) {
+    const void* rk[1] = {a.kw.data + n * row_bytes};
+    const void* rv[1] = {a.vw.data + n * row_bytes};
+    const void* rr[1] = {a.rw.data + n * row_bytes};
+    b.k.load(rk, nchunk, lane);
+    b.v.load(rv, nchunk, lane);
+    b.r.load(rr, nchunk, lane);
+  };
+  Rows3 cur;
   float st_tf = 0.f, st_td = 0.f, st_pp = 0.f, st_aa = 0.f, st_bb = 0.f;
   if (c0 < c1) {
-    const void* rows[3] = {a.kw.data + c0 * row_bytes, a.vw.data + c0 * row_bytes, a.rw.data + c0 * row_bytes};
-    cur.load(rows, nchunk, lane);
+    load3(cur, c0);
   }
 
   // everything the prologue needs from global memory is requested before the layernorm's barriers
@@ -385,16 +368,23 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
     for (int i = 0; i < 3 * kQSums; i++) qt[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tv), i));
   }
 
-  const void* const xv[3] = {kx, vx, rx};
+  // the next channel's rows are requested ahead of the current one's products where two sets of
+  // rows fit in the register file; long rows are loaded one channel at a time
+  constexpr bool kAhead = U8 ? NCH <= 2 : NCH <= 5;
   for (int n = c0; n < c1; n++) {
-    RowBatch<3, NCH, U8> nxt;
-    if (n + 1 < c1) {
-      const void* rows[3] = {a.kw.data + (n + 1) * row_bytes, a.vw.data + (n + 1) * row_bytes,
-                             a.rw.data + (n + 1) * row_bytes};
-      nxt.load(rows, nchunk, lane);
-    }
+    Rows3 nxt;
+    if constexpr (kAhead)
+      if (n + 1 < c1) load3(nxt, n + 1);
     float acc[3];
-    cur.dot(xv, lane, acc);
+    {
+      float t[1];
+      cur.k.dot_shared(kx, lane, t);
+      acc[0] = t[0];
+      cur.v.dot_shared(vx, lane, t);
+      acc[1] = t[0];
+      cur.r.dot_shared(rx, lane, t);
+      acc[2] = t[0];
+    }
     float k = wave_sum(acc[0]);
     float v = wave_sum(acc[1]);
     float rr = wave_sum(acc[2]);
@@ -425,7 +415,12 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       a.bb_out[n] = e1 * bb_ + e2;
       a.pp_out[n] = p_;
     }
-    if (n + 1 < c1) cur = nxt;
+    if (n + 1 < c1) {
+      if constexpr (kAhead)
+        cur = nxt;
+      else
+        load3(cur, n + 1);
+    }
   }
 }
 
@@ -463,7 +458,8 @@ struct RowsArgs {
   Split split;    // rows of all segments over the waves of the grid (set at launch)
   int nseg, nvec; // segments, staged vectors
   int prologue;
-  int start[kMaxSeg + 1];  // first global row of each segment; start[nseg] = total rows
+  int start[kMaxSeg + 1];  // first global row of each segment; start[nseg] = total rows (host bookkeeping)
+  int bstart[kMaxSeg + 1]; // first batch of each segment for the launch's R (set at launch)
   Seg seg[kMaxSeg];
   // prologue inputs
   const h1* vec0;                      // P_COPY
@@ -516,89 +512,54 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   float qtv = 0.f;  // uint8: lane v holds total v of (Sx, Smy) x segments
 
   const int lane = threadIdx.x & (kWave - 1);
-  // The concatenated row space of all segments is split evenly over the waves of the grid;
-  // global row g belongs to the segment s with start[s] <= g < start[s+1].
-  int g0, g1;
-  // The wave index is made visibly uniform: otherwise the per-row lookups in the kernel arguments
+  // Work is dealt in batches of R rows that never straddle two matrices: segment s owns the batches
+  // bstart[s] .. bstart[s+1]-1 (its last batch may be short), and the batches of all segments are
+  // split evenly over the waves of the grid.  One batch therefore multiplies one staged vector.
+  // The wave index is made visibly uniform: otherwise the lookups in the kernel arguments
   // (segment table, row addresses) become vector loads that every weight load has to wait for.
+  int g0, g1;
   split_even(a.split, blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), g0, g1);
 
   struct Meta {
-    int seg[R], loc[R];
-    h1 ex, er;  // epilogue operands of the row this lane finishes (lane < R)
+    int seg, loc0, nvalid;  // segment, first row within it, rows of the batch that exist
   };
-  // locate the rows of the batch starting at global row g and issue their loads
-  auto seg_of = [&](int gg) {
+  // locate batch `bi` and issue the loads of its rows
+  auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int bi) {
     int sg = 0;
 #pragma unroll
-    for (int i = 1; i < kMaxSeg; i++) sg += (i < a.nseg && gg >= a.start[i]) ? 1 : 0;
-    return sg;
-  };
-  auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int g) {
+    for (int i = 1; i < kMaxSeg; i++) sg += (i < a.nseg && bi >= a.bstart[i]) ? 1 : 0;
+    const int n = a.seg[sg].w.N;
+    m.seg = sg;
+    m.loc0 = (bi - a.bstart[sg]) * R;
+    m.nvalid = n - m.loc0 < R ? n - m.loc0 : R;
+    const unsigned char* base = a.seg[sg].w.data;
     const void* rows[R];
-    const int glast = g + R - 1 < g1 ? g + R - 1 : g1 - 1;  // surplus slots re-read the last row
-    const int sg0 = seg_of(g);
-    if (sg0 == seg_of(glast)) {
-      // the usual case, a batch within one matrix: one lookup in the segment table
-      const int loc0 = g - a.start[sg0];
-      const unsigned char* base = a.seg[sg0].w.data;
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        const int gg = g + r < g1 ? g + r : g1 - 1;
-        m.seg[r] = sg0;
-        m.loc[r] = loc0 + (gg - g);
-        rows[r] = base + (size_t)m.loc[r] * row_bytes;
-      }
-    } else {
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        const int gg = g + r < g1 ? g + r : g1 - 1;
-        const int sg = seg_of(gg);
-        m.seg[r] = sg;
-        m.loc[r] = gg - a.start[sg];
-        rows[r] = a.seg[sg].w.data + (size_t)m.loc[r] * row_bytes;
-      }
-    }
-    b.load(rows, nchunk, lane);
-    m.ex = (h1)0.0f;
-    m.er = (h1)0.0f;
-  };
-  auto consume = [&](const RowBatch<R, NCH, U8>& b, const Meta& m, int g) {
-    const void* xv[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      xv[r] = vec_at(U8 ? m.seg[r] : a.seg[m.seg[r]].vec);
+      const int loc = m.loc0 + r < n ? m.loc0 + r : n - 1;  // surplus slots re-read the last row
+      rows[r] = base + (size_t)loc * row_bytes;
     }
+    b.load(rows, nchunk, lane);
+  };
+  auto consume = [&](const RowBatch<R, NCH, U8>& b, const Meta& m) {
+    const Seg& sg = a.seg[m.seg];
     float acc[R];
-    bool same = true;
-#pragma unroll
-    for (int r = 1; r < R; r++) same = same && xv[r] == xv[0];
-    if (same)
-      b.dot_shared(xv[0], lane, acc);  // the usual case: a batch within one matrix
-    else
-      b.dot(xv, lane, acc);
+    b.dot_shared(vec_at(U8 ? m.seg : sg.vec), lane, acc);
     float mine = 0.f;
-    int my_seg = 0, my_loc = 0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
       const float t = wave_sum(acc[r]);
-      if (lane == r) {
-        mine = t;
-        my_seg = m.seg[r];
-        my_loc = m.loc[r];
-      }
+      if (lane == r) mine = t;
     }
-    float q0 = 0.f, q1 = 0.f;
-    if constexpr (U8) {  // lane v holds total v: fetch the two of this lane's segment (all lanes take part)
-      q0 = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (my_seg * kQSums + 0), __float_as_int(qtv)));
-      q1 = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (my_seg * kQSums + 1), __float_as_int(qtv)));
-    }
-    if (lane < R && g + lane < g1) {
+    if (lane < m.nvalid) {
+      const int n = m.loc0 + lane;
       if constexpr (U8) {
-        const WMat& w = a.seg[my_seg].w;
-        mine = finish_q(mine, (float)w.rx[my_loc], (float)w.mx[my_loc], q0, q1);
+        // lane v of qtv holds total v of (Sx, Smy) x segments; the segment is uniform here
+        const float q0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums + 0));
+        const float q1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums + 1));
+        mine = finish_q(mine, (float)sg.w.rx[n], (float)sg.w.mx[n], q0, q1);
       }
-      run_epilogue(a, a.seg[my_seg], my_loc, mine, m.ex, m.er);
+      run_epilogue(a, sg, n, mine, (h1)0.0f, (h1)0.0f);
     }
   };
 
@@ -699,7 +660,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   }
 
   if constexpr (!MULTI) {
-    if (g0 < g1) consume(A, mA, g0);  // the host guarantees g1 - g0 <= R
+    if (g0 < g1) consume(A, mA);  // the host guarantees at most one batch per wave
   } else {
     // Two register sets alternate.  Each "fetch the next, consume the current" pair is straight-line
     // code, so the loads of the next batch stay in flight while the current one is consumed.
@@ -708,20 +669,20 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     int g = g0;
     if (g < g1) {
       for (;;) {
-        if (g + R >= g1) {
-          consume(A, mA, g);
+        if (g + 1 >= g1) {
+          consume(A, mA);
           break;
         }
-        fetch(B, mB, g + R);
-        consume(A, mA, g);
-        g += R;
-        if (g + R >= g1) {
-          consume(B, mB, g);
+        fetch(B, mB, g + 1);
+        consume(A, mA);
+        g += 1;
+        if (g + 1 >= g1) {
+          consume(B, mB);
           break;
         }
-        fetch(A, mA, g + R);
-        consume(B, mB, g);
-        g += R;
+        fetch(A, mA, g + 1);
+        consume(B, mB);
+        g += 1;
       }
     }
   }
@@ -860,21 +821,26 @@ static int env_int(const char* name, int dflt) {
   return (e && atoi(e) > 0) ? atoi(e) : dflt;
 }
 
+// Batches of R rows that never straddle two segments: their number for a given R.
+static long count_batches(const RowsArgs& a, int R) {
+  long nb = 0;
+  for (int s = 0; s < a.nseg; s++) nb += (a.seg[s].w.N + R - 1) / R;
+  return nb;
+}
+
 static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
-  // uint8 rows cost several VALU operations per element: smaller batches let the dequantisation
-  // of one batch overlap the loads of the next
   static const int max_u8 = env_int("FRHIP_MAXLOADS_U8", kMaxLoads);
   const int kMaxLoads = u8 ? max_u8 : frhip::kMaxLoads;
   const long waves = (long)grid * kWaves;
-  long per = ((long)a.start[a.nseg] + waves - 1) / waves;  // most rows any wave gets
-  if (per < 1) per = 1;
   int rmax = kMaxLoads / nch;
   if (rmax < 1) rmax = 1;
   if (rmax > 6) rmax = 6;
-  if (per <= rmax) {
-    *multi = false;
-    return (int)per;
-  }
+  // the smallest R for which every wave gets at most one batch: a single register-resident batch
+  for (int r = 1; r <= rmax; r++)
+    if (count_batches(a, r) <= waves) {
+      *multi = false;
+      return r;
+    }
   *multi = true;
   int r = (kMaxLoads / 2) / nch;
   if (r < 1) r = 1;
@@ -935,9 +901,12 @@ static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char
   if (nch < 0) return set_error(FRHIP_ESHAPE, "K is too large for the row-streaming kernel (max 9216 fp16 / 18432 uint8)");
   const int grid = decode_grid();
   RowsArgs a = args;
-  a.split = make_split(a.start[a.nseg], grid);
   bool multi = false;
   const int R = pick_r(a, grid, nch, u8, &multi);
+  a.bstart[0] = 0;
+  for (int s = 0; s < kMaxSeg; s++)
+    a.bstart[s + 1] = s < a.nseg ? a.bstart[s] + (a.seg[s].w.N + R - 1) / R : INT_MAX;
+  a.split = make_split(a.bstart[a.nseg], grid);
   const size_t lds = staged_bytes(nch, u8) * (u8 ? a.nseg : a.nvec);
   FR_TRY(check_lds(lds));
   bool ok = false;
