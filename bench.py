@@ -256,6 +256,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the int8-decode and prefill side measurements")
     ap.add_argument("--probe", action="store_true", help="only run the read/copy bandwidth probes and print them")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only run the T=1024 seq-mode prefill side measurement and print it (profiling aid)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs batch-1 decode on ONE GPU; --gpus %d is not supported "
@@ -266,6 +268,9 @@ def main():
     fr = importlib.import_module("faster-rwkv_amd")
     if args.probe:
         print(json.dumps(probe_bandwidth(fr)), flush=True)
+        return
+    if args.prefill_only:
+        print(json.dumps(prefill_extra(fr)), flush=True)
         return
     cfg = CONFIGS[args.dtype]
     t0 = time.perf_counter()
