@@ -68,41 +68,33 @@ struct LnOut {
 };
 
 // `red` holds 2 * kWaves floats: the two reductions use separate halves, one barrier each.
-__device__ __forceinline__ LnOut ln_block(const h1* x, const h1* gamma, const h1* beta, int C, float* red) {
-  const int e0 = threadIdx.x * 8;
+// The thread's eight elements and their gamma / beta arrive in registers: callers request them
+// ahead of the weight rows, so that the normalisation runs while the rows are in flight
+// (vector loads return in the order they were issued).
+__device__ __forceinline__ LnOut ln_regs(h8 xv, h8 g, h8 b, bool active, int C, float* red) {
   LnOut o;
-  o.active = e0 < C;
+  o.active = active;
   float xf[8];
   float s = 0.f;
-  h8 g, b;
-  if (o.active) {
-    h8 xv = *reinterpret_cast<const h8*>(x + e0);
-    g = *reinterpret_cast<const h8*>(gamma + e0);
-    b = *reinterpret_cast<const h8*>(beta + e0);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      xf[i] = (float)xv[i];
-      s += xf[i];
-    }
+  for (int i = 0; i < 8; i++) {
+    xf[i] = active ? (float)xv[i] : 0.f;
+    s += xf[i];
   }
   const float mean = block_sum1<kWaves>(s, red) / (float)C;
   float q = 0.f;
-  if (o.active) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      float d = xf[i] - mean;
-      q += d * d;
-    }
+  for (int i = 0; i < 8; i++) {
+    float d = xf[i] - mean;
+    q += active ? d * d : 0.f;
   }
   float var = block_sum1<kWaves>(q, red + kWaves) / (float)C;
   var = var > 0.f ? var : 0.f;
   const float inv = 1.0f / sqrtf(var + 1e-5f);
-  if (o.active) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      h1 n = (h1)((xf[i] - mean) * inv);
-      o.xx[i] = (n * g[i]) + b[i];
-    }
+  for (int i = 0; i < 8; i++) {
+    h1 n = (h1)((xf[i] - mean) * inv);
+    o.xx[i] = (n * g[i]) + b[i];
   }
   return o;
 }
@@ -140,14 +132,23 @@ struct RowBatch {
   static constexpr int kPadChunks = NCH * kWave;  // chunks per staged vector, padding included
   V w[R][NCH];
 
-  __device__ __forceinline__ void load(const void* const (&rows)[R], int nchunk, int lane) {
+  // Rows are read through buffer descriptors (base = start of the row, extent = nbytes[r]): a
+  // lane whose chunk lies beyond the extent gets zeros without a memory access, which serves
+  // the tail of a row whose length is not a multiple of 64 chunks, the surplus slots of a short
+  // batch and waves without work (extent 0) alike, with the same number of loads issued.
+  __device__ __forceinline__ void load(const void* const (&rows)[R], const int (&nbytes)[R], int lane) {
+    __amdgpu_buffer_rsrc_t rs[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
+    for (int r = 0; r < R; r++)
+      rs[r] = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(rows[r]), 0, nbytes[r], 0x00020000);
+    // chunk-major, the order in which dot_shared() consumes them
 #pragma unroll
-      for (int j = 0; j < NCH; j++) {
-        int c = lane + j * kWave;
-        c = c < nchunk ? c : nchunk - 1;
-        w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const V*>(rows[r]) + c);
+    for (int j = 0; j < NCH; j++) {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs[r], lane * 16 + (j & 3) * (kWave * 16),
+                                                              (j >> 2) * (4 * kWave * 16), 2 /* nontemporal */);
+        w[r][j] = __builtin_bit_cast(V, v);
       }
     }
   }
@@ -283,10 +284,15 @@ struct AttFrontV4 {
   float *aa_out, *bb_out, *pp_out;
 };
 
-template <int NCH, bool U8>
+// SINGLE: no wave owns more than one channel (the host checks).  That kernel has no loop and no
+// second set of rows, so nothing competes with the loads in flight for registers.
+template <int NCH, bool U8, bool SINGLE>
 __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float red[2 * kWaves];
+  // One field from every 64-byte line of the kernel arguments is requested up front, so that the
+  // scalar loads further down (issued where each field is first needed) hit the scalar cache.
+  asm volatile("" ::"s"(a.C), "s"(a.tf), "s"(a.vw.data), "s"(a.rw.data), "s"(a.xx_out));
   const int C = a.C;
   const int nchunk = U8 ? (C >> 4) : (C >> 3);
   // binary16: the three mixed vectors; uint8: the three pre-scaled fp32 vectors xr (see stage_q)
@@ -308,25 +314,30 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   struct Rows3 {
     RowBatch<1, NCH, U8> k, v, r;
   };
-  auto load3 = [&](Rows3& b, int n) {
+  auto load3 = [&](Rows3& b, int n, bool live) {
     const void* rk[1] = {a.kw.data + n * row_bytes};
     const void* rv[1] = {a.vw.data + n * row_bytes};
     const void* rr[1] = {a.rw.data + n * row_bytes};
-    b.k.load(rk, nchunk, lane);
-    b.v.load(rv, nchunk, lane);
-    b.r.load(rr, nchunk, lane);
+    const int nb[1] = {live ? (int)row_bytes : 0};
+    b.k.load(rk, nb, lane);
+    b.v.load(rv, nb, lane);
+    b.r.load(rr, nb, lane);
   };
-  Rows3 cur;
-  float st_tf = 0.f, st_td = 0.f, st_pp = 0.f, st_aa = 0.f, st_bb = 0.f;
-  if (c0 < c1) {
-    load3(cur, c0);
-  }
-
-  // everything the prologue needs from global memory is requested before the layernorm's barriers
+  // Every global operand is requested before the first wait, operands of the prologue first: the
+  // layernorm and the staging then run while the weight rows are in flight, and the products
+  // start on the first chunks that arrive (vector loads return in the order they were issued).
+  // The rows are loaded unconditionally and last (waves without a channel read a valid
+  // duplicate): a load inside a branch after them would make the number of loads in flight
+  // path-dependent and every later wait a wait for all of them.  Before them branches are
+  // harmless, and only threads that own a group load: every byte requested here passes through
+  // the compute unit's vector memory pipeline ahead of the rows.
   const bool own = (int)threadIdx.x * 8 < C;
   const int e0 = threadIdx.x * 8;
-  h8 sx, mixk, mixv, mixr, qry[3], qmy[3];
+  h8 xv{}, lg{}, lb{}, sx{}, mixk{}, mixv{}, mixr{}, qry[3] = {}, qmy[3] = {};
   if (own) {
+    xv = *reinterpret_cast<const h8*>(a.x + e0);
+    lg = *reinterpret_cast<const h8*>(a.ln_w + e0);
+    lb = *reinterpret_cast<const h8*>(a.ln_b + e0);
     sx = *reinterpret_cast<const h8*>(a.sx + e0);
     mixk = *reinterpret_cast<const h8*>(a.mk + e0);
     mixv = *reinterpret_cast<const h8*>(a.mv + e0);
@@ -337,7 +348,28 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       qry[2] = *reinterpret_cast<const h8*>(a.rw.ry + e0); qmy[2] = *reinterpret_cast<const h8*>(a.rw.my + e0);
     }
   }
-  LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, C, red);
+  // recurrent state and per-row constants of a channel (every lane reads the same words)
+  struct Chan {
+    float tf, td, pp, aa, bb;
+    h1 qrx[3], qmx[3];
+  };
+  auto load_chan = [&](Chan& s, int n) {
+    s.tf = a.tf[n]; s.td = a.td[n]; s.pp = a.pp[n]; s.aa = a.aa[n]; s.bb = a.bb[n];
+    if constexpr (U8) {
+      s.qrx[0] = a.kw.rx[n]; s.qmx[0] = a.kw.mx[n];
+      s.qrx[1] = a.vw.rx[n]; s.qmx[1] = a.vw.mx[n];
+      s.qrx[2] = a.rw.rx[n]; s.qmx[2] = a.rw.mx[n];
+    }
+  };
+  Rows3 cur;
+  Chan st;
+  {
+    const int first = c0 < c1 ? c0 : C - 1;
+    load_chan(st, first);
+    load3(cur, first, c0 < c1);
+  }
+
+  LnOut ln = ln_regs(xv, lg, lb, own, C, red);
   float part[3 * kQSums];
 #pragma unroll
   for (int i = 0; i < 3 * kQSums; i++) part[i] = 0.f;
@@ -368,46 +400,38 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
     for (int i = 0; i < 3 * kQSums; i++) qt[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tv), i));
   }
 
-  // the next channel's rows are requested ahead of the current one's products where two sets of
-  // rows fit in the register file; long rows are loaded one channel at a time
-  constexpr bool kAhead = U8 ? NCH <= 2 : NCH <= 5;
-  for (int n = c0; n < c1; n++) {
-    Rows3 nxt;
-    if constexpr (kAhead)
-      if (n + 1 < c1) load3(nxt, n + 1);
+  // products, reduction and state update of one channel whose rows and state are in registers
+  auto channel = [&](int n, const Rows3& rows, const Chan& st) {
     float acc[3];
     {
       float t[1];
-      cur.k.dot_shared(kx, lane, t);
+      rows.k.dot_shared(kx, lane, t);
       acc[0] = t[0];
-      cur.v.dot_shared(vx, lane, t);
+      rows.v.dot_shared(vx, lane, t);
       acc[1] = t[0];
-      cur.r.dot_shared(rx, lane, t);
+      rows.r.dot_shared(rx, lane, t);
       acc[2] = t[0];
     }
     float k = wave_sum(acc[0]);
     float v = wave_sum(acc[1]);
     float rr = wave_sum(acc[2]);
     if constexpr (U8) {
-      k = finish_q(k, (float)a.kw.rx[n], (float)a.kw.mx[n], qt[0], qt[1]);
-      v = finish_q(v, (float)a.vw.rx[n], (float)a.vw.mx[n], qt[2], qt[3]);
-      rr = finish_q(rr, (float)a.rw.rx[n], (float)a.rw.mx[n], qt[4], qt[5]);
+      k = finish_q(k, (float)st.qrx[0], (float)st.qmx[0], qt[0], qt[1]);
+      v = finish_q(v, (float)st.qrx[1], (float)st.qmx[1], qt[2], qt[3]);
+      rr = finish_q(rr, (float)st.qrx[2], (float)st.qmx[2], qt[4], qt[5]);
     }
     if (lane == 0) {
       // kernels/cuda/att.cu:30-62 (WkvForwardOne), r already passed through sigmoid (:203)
-      {
-        st_tf = a.tf[n]; st_td = a.td[n]; st_pp = a.pp[n]; st_aa = a.aa[n]; st_bb = a.bb[n];
-      }
       const h1 r = sigmoid_h((h1)rr);
-      float ww = st_tf + k;
-      const float pp_ = st_pp;
+      float ww = st.tf + k;
+      const float pp_ = st.pp;
       float p_ = (pp_ > ww) ? pp_ : ww;
       float e1 = expf(pp_ - p_);
       float e2 = expf(ww - p_);
-      const float aa_ = st_aa, bb_ = st_bb;
+      const float aa_ = st.aa, bb_ = st.bb;
       const float wkv = (e1 * aa_ + e2 * v) / (e1 * bb_ + e2);
       a.rwkv_out[n] = r * (h1)wkv;
-      ww = st_td + pp_;
+      ww = st.td + pp_;
       p_ = (ww > k) ? ww : k;
       e1 = expf(ww - p_);
       e2 = expf(k - p_);
@@ -415,11 +439,34 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       a.bb_out[n] = e1 * bb_ + e2;
       a.pp_out[n] = p_;
     }
+  };
+
+  if constexpr (SINGLE) {
+    // no load follows the rows: every wait for a chunk is exact
+    if (c0 < c1) channel(c0, cur, st);
+    return;
+  }
+  // Several channels per wave: the next channel's rows are requested ahead of the current one's
+  // products where two sets of rows fit in the register file; long rows are loaded one channel
+  // at a time.
+  constexpr bool kAhead = U8 ? NCH <= 2 : NCH <= 5;
+  for (int n = c0; n < c1; n++) {
+    Rows3 nxt;
+    Chan nst;
+    if constexpr (kAhead)
+      if (n + 1 < c1) {
+        load_chan(nst, n + 1);
+        load3(nxt, n + 1, true);
+      }
+    channel(n, cur, st);
     if (n + 1 < c1) {
-      if constexpr (kAhead)
+      if constexpr (kAhead) {
         cur = nxt;
-      else
-        load3(cur, n + 1);
+        st = nst;
+      } else {
+        load_chan(st, n + 1);
+        load3(cur, n + 1, true);
+      }
     }
   }
 }
@@ -469,6 +516,7 @@ struct RowsArgs {
   // epilogue inputs
   const h1* res_x;  // E_RESIDUAL, E_FFN_OUT
   const h1* res_r;  // E_FFN_OUT
+  int res_n;        // elements of res_x / res_r that may be read (1 when no epilogue uses them)
   int div2;
 };
 
@@ -476,7 +524,7 @@ __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, i
   switch (sg.epi) {
     case E_STORE_F16: static_cast<h1*>(sg.out)[n] = (h1)sum; break;
     case E_STORE_F32: static_cast<float*>(sg.out)[n] = sum; break;
-    case E_RESIDUAL: static_cast<h1*>(sg.out)[n] = a.res_x[n] + (h1)sum; break;
+    case E_RESIDUAL: static_cast<h1*>(sg.out)[n] = ex + (h1)sum; break;
     case E_SIGMOID: static_cast<h1*>(sg.out)[n] = sigmoid_h((h1)sum); break;
     case E_RELU2: {
       h1 t = (h1)sum;
@@ -484,7 +532,7 @@ __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, i
       break;
     }
     case E_FFN_OUT: {
-      h1 o = __builtin_fmaf16((h1)sum, a.res_r[n], a.res_x[n]);  // __hfma: one rounding
+      h1 o = __builtin_fmaf16((h1)sum, er, ex);  // __hfma: one rounding
       if (a.div2) o = o / (h1)2.0f;
       static_cast<h1*>(sg.out)[n] = o;
       break;
@@ -497,10 +545,22 @@ __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, i
 
 // MULTI = a wave has several batches: two batches live in registers and alternate, the
 // loads of one in flight while the other is consumed.
-template <int R, int NCH, bool U8, bool MULTI>
+// PRO = the prologue, known at compile time so that its loads form straight-line code.
+//
+// Order of the global loads: operands of the prologue, then the first batch of rows with the
+// per-row operands of its epilogue, all before the first wait and none inside a branch (threads
+// and waves without work read a valid duplicate).  Vector loads return in the order they were
+// issued, so the prologue runs while the rows are in flight and the products start on the
+// first chunks that arrive; a load inside a branch would make the number of loads in flight
+// path-dependent and turn every later wait into a wait for all of them.
+template <int R, int NCH, bool U8, bool MULTI, int PRO>
 __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float red[2 * kWaves];
+  // One field from every 64-byte line of the kernel arguments is requested up front, so that the
+  // scalar loads further down (issued where each field is first needed) hit the scalar cache.
+  asm volatile("" ::"s"(a.K), "s"(a.seg[0].out), "s"(a.seg[1].out), "s"(a.seg[2].out), "s"(a.seg[3].out), "s"(a.vec0),
+               "s"(a.res_x));
   const int K = a.K;
   const int nchunk = U8 ? (K >> 4) : (K >> 3);
   const size_t row_bytes = U8 ? (size_t)K : 2 * (size_t)K;
@@ -522,9 +582,17 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
 
   struct Meta {
     int seg, loc0, nvalid;  // segment, first row within it, rows of the batch that exist
+    // Per-row operands of the epilogue, lane r holding those of row r.  They are requested with the
+    // batch's weights: asked for after the products they would cost a whole memory latency at the
+    // end of the launch.
+    h1 ex, er, qrx, qmx;
   };
-  // locate batch `bi` and issue the loads of its rows
-  auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int bi) {
+  // Row addresses and extents of a batch; `live` = the batch is this wave's to finish.
+  struct Where {
+    const void* rows[R];
+    int nbytes[R];
+  };
+  auto locate = [&](Meta& m, Where& wh, int bi, bool live) {
     int sg = 0;
 #pragma unroll
     for (int i = 1; i < kMaxSeg; i++) sg += (i < a.nseg && bi >= a.bstart[i]) ? 1 : 0;
@@ -532,14 +600,35 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     m.seg = sg;
     m.loc0 = (bi - a.bstart[sg]) * R;
     m.nvalid = n - m.loc0 < R ? n - m.loc0 : R;
+    if (!live) m.nvalid = 0;
     const unsigned char* base = a.seg[sg].w.data;
-    const void* rows[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const int loc = m.loc0 + r < n ? m.loc0 + r : n - 1;  // surplus slots re-read the last row
-      rows[r] = base + (size_t)loc * row_bytes;
+      const bool have = live && m.loc0 + r < n;  // surplus slots and idle waves read nothing
+      wh.rows[r] = base + (size_t)(have ? m.loc0 + r : 0) * row_bytes;
+      wh.nbytes[r] = have ? (int)row_bytes : 0;
     }
-    b.load(rows, nchunk, lane);
+  };
+  // issue the loads of a located batch: its rows, then the per-row operands of its epilogue
+  auto request = [&](RowBatch<R, NCH, U8>& b, Meta& m, const Where& wh) {
+    b.load(wh.rows, wh.nbytes, lane);
+    const int n = a.seg[m.seg].w.N;
+    const int nl = m.loc0 + lane < n ? m.loc0 + lane : n - 1;
+    m.ex = m.er = (h1)0.0f;
+    if constexpr (PRO == P_COPY) {  // the launches with residual epilogues all stage a ready vector
+      const int ri = nl < a.res_n ? nl : a.res_n - 1;
+      m.ex = a.res_x[ri];
+      m.er = a.res_r[ri];
+    }
+    if constexpr (U8) {
+      m.qrx = a.seg[m.seg].w.rx[nl];
+      m.qmx = a.seg[m.seg].w.mx[nl];
+    }
+  };
+  auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int bi, bool live) {
+    Where wh;
+    locate(m, wh, bi, live);
+    request(b, m, wh);
   };
   auto consume = [&](const RowBatch<R, NCH, U8>& b, const Meta& m) {
     const Seg& sg = a.seg[m.seg];
@@ -557,100 +646,109 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
         // lane v of qtv holds total v of (Sx, Smy) x segments; the segment is uniform here
         const float q0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums + 0));
         const float q1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums + 1));
-        mine = finish_q(mine, (float)sg.w.rx[n], (float)sg.w.mx[n], q0, q1);
+        mine = finish_q(mine, (float)m.qrx, (float)m.qmx, q0, q1);
       }
-      run_epilogue(a, sg, n, mine, (h1)0.0f, (h1)0.0f);
+      run_epilogue(a, sg, n, mine, m.ex, m.er);
     }
   };
 
-  RowBatch<R, NCH, U8> A;
+  // where the first batch lives: scalar work, done before any load is requested
   Meta mA;
-  if (g0 < g1) fetch(A, mA, g0);
+  Where whA;
+  locate(mA, whA, g0 < g1 ? g0 : a.bstart[a.nseg] - 1, g0 < g1);
 
-  // ---- prologue: stage the activation vector(s) in LDS ----
-  // Global operands of the prologue are requested before the layernorm's barriers.
-  {
-    const int e0 = threadIdx.x * 8;
-    const bool own = a.prologue != P_COPY && e0 < K;
-    h8 sx, mixv[kMaxSeg], qry[kMaxSeg], qmy[kMaxSeg];
-    if (own) {
-      if (a.prologue == P_LN_MIX) {
-        sx = *reinterpret_cast<const h8*>(a.sx + e0);
+  // ---- operands of the prologue ----
+  // P_COPY: the vector (one segment; uint8: with its ry, my) in passes of one 8-element group per
+  // thread; P_LN / P_LN_MIX: K <= 8 * kThreads, one group per thread.  Only threads that own a
+  // group load (every byte requested here passes through the compute unit's vector memory
+  // pipeline ahead of the rows): branches are harmless before the rows, whose count is fixed.
+  constexpr int kCopyPasses = (NCH * kWave * (U8 ? 2 : 1) + kThreads - 1) / kThreads;
+  const int ngrp = K >> 3;
+  const bool own = (int)threadIdx.x < ngrp;
+  const int e0 = threadIdx.x * 8;
+  h8 cx[kCopyPasses] = {}, cry[kCopyPasses] = {}, cmy[kCopyPasses] = {};
+  h8 xv{}, lg{}, lb{}, sxv{}, mixv[kMaxSeg] = {}, qry[kMaxSeg] = {}, qmy[kMaxSeg] = {};
+  if constexpr (PRO == P_COPY) {
 #pragma unroll
-        for (int i = 0; i < kMaxSeg; i++)
-          if (i < a.nvec) mixv[i] = *reinterpret_cast<const h8*>(a.mix[i] + e0);
-      }
-      if constexpr (U8) {
-#pragma unroll
-        for (int i = 0; i < kMaxSeg; i++)
-          if (i < a.nseg) {
-            qry[i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + e0);
-            qmy[i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + e0);
-          }
+    for (int p = 0; p < kCopyPasses; p++) {
+      const int g = (int)threadIdx.x + p * kThreads;
+      if (g < ngrp) {
+        cx[p] = reinterpret_cast<const h8*>(a.vec0)[g];
+        if constexpr (U8) {
+          cry[p] = reinterpret_cast<const h8*>(a.seg[0].w.ry)[g];
+          cmy[p] = reinterpret_cast<const h8*>(a.seg[0].w.my)[g];
+        }
       }
     }
+  } else if (own) {
+    xv = *reinterpret_cast<const h8*>(a.x + e0);
+    lg = *reinterpret_cast<const h8*>(a.ln_w + e0);
+    lb = *reinterpret_cast<const h8*>(a.ln_b + e0);
+    if constexpr (PRO == P_LN_MIX) {
+      sxv = *reinterpret_cast<const h8*>(a.sx + e0);
+#pragma unroll
+      for (int i = 0; i < kMaxSeg; i++)
+        if (i < a.nvec) mixv[i] = *reinterpret_cast<const h8*>(a.mix[i] + e0);
+    }
+    if constexpr (U8) {
+#pragma unroll
+      for (int i = 0; i < kMaxSeg; i++)
+        if (i < a.nseg) {
+          qry[i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + e0);
+          qmy[i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + e0);
+        }
+    }
+  }
+
+  // ---- first batch of rows ----
+  RowBatch<R, NCH, U8> A;
+  request(A, mA, whA);
+
+  // ---- prologue: stage the activation vector(s) in LDS ----
+  {
     float part[kMaxSeg * kQSums];
 #pragma unroll
     for (int i = 0; i < kMaxSeg * kQSums; i++) part[i] = 0.f;
-    if (a.prologue == P_COPY) {
-      if constexpr (!U8) {
-        stage_vec<false>(reinterpret_cast<h1*>(vec_at(0)), a.vec0, K);
-      } else {
-        // two groups per thread and pass, every load of a pass requested before its first use
-        const int ngrp = K >> 3;
-        for (int g = threadIdx.x; g < ngrp; g += 2 * kThreads) {
-          const int g2 = g + kThreads;
-          const bool two = g2 < ngrp;
-          h8 x[2], ry[2][kMaxSeg], my[2][kMaxSeg];
-          x[0] = reinterpret_cast<const h8*>(a.vec0)[g];
-          if (two) x[1] = reinterpret_cast<const h8*>(a.vec0)[g2];
+    if constexpr (PRO == P_COPY) {
 #pragma unroll
-          for (int i = 0; i < kMaxSeg; i++)
-            if (i < a.nseg) {
-              ry[0][i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + 8 * g);
-              my[0][i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + 8 * g);
-              if (two) {
-                ry[1][i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + 8 * g2);
-                my[1][i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + 8 * g2);
-              }
-            }
-#pragma unroll
-          for (int i = 0; i < kMaxSeg; i++)
-            if (i < a.nseg) {
-              stage_q(reinterpret_cast<float*>(vec_at(i)), g, kPad, x[0], ry[0][i], my[0][i], part + i * kQSums);
-              if (two) stage_q(reinterpret_cast<float*>(vec_at(i)), g2, kPad, x[1], ry[1][i], my[1][i], part + i * kQSums);
-            }
+      for (int p = 0; p < kCopyPasses; p++) {
+        const int g = (int)threadIdx.x + p * kThreads;
+        if (g < ngrp) {
+          if constexpr (!U8)
+            reinterpret_cast<h8*>(vec_at(0))[g] = cx[p];
+          else
+            stage_q(reinterpret_cast<float*>(vec_at(0)), g, kPad, cx[p], cry[p], cmy[p], part);
         }
       }
     } else {
-      LnOut ln = ln_block(a.x, a.ln_w, a.ln_b, K, red);
+      LnOut ln = ln_regs(xv, lg, lb, own, K, red);
       if (ln.active) {
         if constexpr (!U8) {
-          if (a.prologue == P_LN) {
+          if constexpr (PRO == P_LN) {
             reinterpret_cast<h8*>(vec_at(0))[threadIdx.x] = ln.xx;
           } else {
 #pragma unroll
             for (int i = 0; i < kMaxSeg; i++)
-              if (i < a.nvec) reinterpret_cast<h8*>(vec_at(i))[threadIdx.x] = mix8(ln.xx, sx, mixv[i]);
+              if (i < a.nvec) reinterpret_cast<h8*>(vec_at(i))[threadIdx.x] = mix8(ln.xx, sxv, mixv[i]);
           }
         } else {
 #pragma unroll
           for (int i = 0; i < kMaxSeg; i++) {
             if (i < a.nseg) {
               h8 x = ln.xx;
-              if (a.prologue == P_LN_MIX) {
+              if constexpr (PRO == P_LN_MIX) {
                 // segment i multiplies staged vector seg[i].vec; pick its mix without dynamic register indexing
                 h8 mx8 = mixv[0];
 #pragma unroll
                 for (int j = 1; j < kMaxSeg; j++)
                   if (a.seg[i].vec == j) mx8 = mixv[j];
-                x = mix8(ln.xx, sx, mx8);
+                x = mix8(ln.xx, sxv, mx8);
               }
               stage_q(reinterpret_cast<float*>(vec_at(i)), threadIdx.x, kPad, x, qry[i], qmy[i], part + i * kQSums);
             }
           }
         }
-        if (a.prologue == P_LN_MIX && blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
+        if (PRO == P_LN_MIX && blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
       }
     }
     for (int i = 0; i < (U8 ? a.nseg : a.nvec); i++) zero_pad<U8>(vec_at(i), nchunk, kPad);
@@ -660,7 +758,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   }
 
   if constexpr (!MULTI) {
-    if (g0 < g1) consume(A, mA);  // the host guarantees at most one batch per wave
+    consume(A, mA);  // the host guarantees at most one batch per wave
   } else {
     // Two register sets alternate.  Each "fetch the next, consume the current" pair is straight-line
     // code, so the loads of the next batch stay in flight while the current one is consumed.
@@ -673,14 +771,14 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
           consume(A, mA);
           break;
         }
-        fetch(B, mB, g + 1);
+        fetch(B, mB, g + 1, true);
         consume(A, mA);
         g += 1;
         if (g + 1 >= g1) {
           consume(B, mB);
           break;
         }
-        fetch(A, mA, g + 1);
+        fetch(A, mA, g + 1, true);
         consume(B, mB);
         g += 1;
       }
@@ -851,26 +949,35 @@ static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
 }
 
 // false when the (R, NCH, MULTI) tiling is not compiled (pick_r never asks for one that is not)
+template <int R, int NCH, bool U8, bool MULTI>
+static void launch_rows_pro(int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
+  switch (a.prologue) {
+    case P_COPY: hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_COPY>), dim3(grid), dim3(kThreads), lds, st, a); break;
+    case P_LN: hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_LN>), dim3(grid), dim3(kThreads), lds, st, a); break;
+    default: hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_LN_MIX>), dim3(grid), dim3(kThreads), lds, st, a); break;
+  }
+}
+
 template <int R, int NCH>
 static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
   if (!multi) {
     if constexpr ((R * NCH <= kMaxLoads && R <= 6) || R == 1) {
       if (u8)
-        hipLaunchKernelGGL((rows_kernel<R, NCH, true, false>), dim3(grid), dim3(kThreads), lds, st, a);
+        launch_rows_pro<R, NCH, true, false>(grid, lds, st, a);
       else
-        hipLaunchKernelGGL((rows_kernel<R, NCH, false, false>), dim3(grid), dim3(kThreads), lds, st, a);
+        launch_rows_pro<R, NCH, false, false>(grid, lds, st, a);
       return true;
     }
   } else {
     if constexpr ((R * NCH <= kMaxLoads / 2 && R <= 4) || R == 1) {
       if (u8)
-        hipLaunchKernelGGL((rows_kernel<R, NCH, true, true>), dim3(grid), dim3(kThreads), lds, st, a);
+        launch_rows_pro<R, NCH, true, true>(grid, lds, st, a);
       else
-        hipLaunchKernelGGL((rows_kernel<R, NCH, false, true>), dim3(grid), dim3(kThreads), lds, st, a);
+        launch_rows_pro<R, NCH, false, true>(grid, lds, st, a);
       return true;
     } else if constexpr (R == 8 && NCH <= 2) {
       if (!u8) return false;
-      hipLaunchKernelGGL((rows_kernel<R, NCH, true, true>), dim3(grid), dim3(kThreads), lds, st, a);
+      launch_rows_pro<R, NCH, true, true>(grid, lds, st, a);
       return true;
     }
   }
@@ -901,6 +1008,15 @@ static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char
   if (nch < 0) return set_error(FRHIP_ESHAPE, "K is too large for the row-streaming kernel (max 9216 fp16 / 18432 uint8)");
   const int grid = decode_grid();
   RowsArgs a = args;
+  // epilogue operands are read unconditionally: point unused ones at any readable element
+  if (!a.res_x || !a.res_r) {
+    const h1* any = reinterpret_cast<const h1*>(a.seg[0].w.data);
+    if (!a.res_x && !a.res_r) a.res_n = 1;
+    if (!a.res_x) a.res_x = a.res_r ? a.res_r : any;
+    if (!a.res_r) a.res_r = a.res_x;
+  }
+  if (a.prologue == P_COPY && a.nseg != 1)
+    return set_error(FRHIP_EINVAL, "row-streaming kernel: a staged ready vector serves one matrix");
   bool multi = false;
   const int R = pick_r(a, grid, nch, u8, &multi);
   a.bstart[0] = 0;
@@ -1028,12 +1144,17 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   const int nch_t = nch <= 1 ? 1 : nch == 2 ? 2 : nch <= 4 ? 4 : nch == 5 ? 5 : 8;  // compiled tilings
   const size_t lds = staged_bytes(nch_t, u8) * 3;
   FR_TRY(check_lds(lds));
+  const bool single = C <= grid * kWaves;
 #define FR_ATT_FRONT(N)                                                                                   \
   do {                                                                                                    \
-    if (u8)                                                                                               \
-      hipLaunchKernelGGL((att_front_v4_kernel<N, true>), dim3(grid), dim3(kThreads), lds, st, a);         \
+    if (u8 && single)                                                                                     \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, true, true>), dim3(grid), dim3(kThreads), lds, st, a);   \
+    else if (u8)                                                                                          \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, true, false>), dim3(grid), dim3(kThreads), lds, st, a);  \
+    else if (single)                                                                                      \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, false, true>), dim3(grid), dim3(kThreads), lds, st, a);  \
     else                                                                                                  \
-      hipLaunchKernelGGL((att_front_v4_kernel<N, false>), dim3(grid), dim3(kThreads), lds, st, a);        \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, false, false>), dim3(grid), dim3(kThreads), lds, st, a); \
   } while (0)
   if (nch <= 1) FR_ATT_FRONT(1);
   else if (nch == 2) FR_ATT_FRONT(2);
@@ -1048,6 +1169,7 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   b.nvec = 1;
   b.vec0 = w.rwkv;
   b.res_x = (const h1*)x;
+  b.res_n = C;
   add_seg(b, ow, 0, E_RESIDUAL, x_out);
   return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_out");
 }
@@ -1110,6 +1232,7 @@ static int att_one_v5_impl(bool v50, int C, int H, const void* x, const void* sx
   b.nvec = 1;
   b.vec0 = w.rwkv;
   b.res_x = (const h1*)x;
+  b.res_n = C;
   add_seg(b, ow, 0, E_RESIDUAL, x_out);
   return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_v5_out");
 }
@@ -1174,6 +1297,7 @@ extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const 
   b.nvec = 1;
   b.vec0 = w.vx;
   b.res_x = (const h1*)x;
+  b.res_n = C;
   b.res_r = w.r;
   b.div2 = post_div2 ? 1 : 0;
   add_seg(b, vw, 0, E_FFN_OUT, x_out);
