@@ -136,14 +136,15 @@ struct RowBatch {
   // lane whose chunk lies beyond the extent gets zeros without a memory access, which serves
   // the tail of a row whose length is not a multiple of 64 chunks, the surplus slots of a short
   // batch and waves without work (extent 0) alike, with the same number of loads issued.
+  template <int J0 = 0, int J1 = NCH>
   __device__ __forceinline__ void load(const void* const (&rows)[R], const int (&nbytes)[R], int lane) {
     __amdgpu_buffer_rsrc_t rs[R];
 #pragma unroll
     for (int r = 0; r < R; r++)
       rs[r] = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(rows[r]), 0, nbytes[r], 0x00020000);
-    // chunk-major, the order in which dot_shared() consumes them
+    // chunk-major, the order in which dot_shared() consumes them; chunks J0 .. J1-1 only
 #pragma unroll
-    for (int j = 0; j < NCH; j++) {
+    for (int j = J0; j < J1; j++) {
 #pragma unroll
       for (int r = 0; r < R; r++) {
         const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs[r], lane * 16 + (j & 3) * (kWave * 16),
@@ -152,6 +153,16 @@ struct RowBatch {
       }
     }
   }
+
+  // Chunks of a batch requested ahead of the prologue.  A compute unit keeps only so many bytes of
+  // loads in flight (about 64 KB: 8 per wave); a wave that asks for more is held at the load
+  // instruction until earlier data has returned, and the older four waves of a workgroup go first.
+  // A prologue that sits behind all loads of a large batch therefore runs when most rows have
+  // arrived (its barriers wait for the last wave to get through its loads).  Batches of more than
+  // 16 loads put about 8 of them first, then the prologue, then the rest; for smaller ones holding
+  // loads back only idles the memory (measured: 24 loads, 6 first: 9.60 -> 9.33 us; 16 loads, 8
+  // first: 7.11 -> 7.32 us; 12 loads, 6 first: 6.81 -> 7.12 us).
+  static constexpr int kHead = R * NCH <= 16 ? NCH : (8 / R < 1 ? 1 : 8 / R);
 
   // All rows against one staged vector, each chunk of which is read from LDS once.  Binary16 rows:
   // acc[r] = sum_k w[k] x[k] against a binary16 vector; uint8 rows: acc[r] = sum_k q[k] xr[k]
@@ -314,15 +325,20 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   struct Rows3 {
     RowBatch<1, NCH, U8> k, v, r;
   };
-  auto load3 = [&](Rows3& b, int n, bool live) {
+  // chunks J0 .. J1-1 of the three rows of channel n
+  auto load3_part = [&](Rows3& b, int n, bool live, auto j0, auto j1) {
     const void* rk[1] = {a.kw.data + n * row_bytes};
     const void* rv[1] = {a.vw.data + n * row_bytes};
     const void* rr[1] = {a.rw.data + n * row_bytes};
     const int nb[1] = {live ? (int)row_bytes : 0};
-    b.k.load(rk, nb, lane);
-    b.v.load(rv, nb, lane);
-    b.r.load(rr, nb, lane);
+    b.k.template load<decltype(j0)::value, decltype(j1)::value>(rk, nb, lane);
+    b.v.template load<decltype(j0)::value, decltype(j1)::value>(rv, nb, lane);
+    b.r.template load<decltype(j0)::value, decltype(j1)::value>(rr, nb, lane);
   };
+  using J0 = std::integral_constant<int, 0>;
+  using JH = std::integral_constant<int, RowBatch<3, NCH, U8>::kHead>;  // requested ahead of the prologue
+  using JN = std::integral_constant<int, NCH>;
+  auto load3 = [&](Rows3& b, int n, bool live) { load3_part(b, n, live, J0{}, JN{}); };
   // Every global operand is requested before the first wait, operands of the prologue first: the
   // layernorm and the staging then run while the weight rows are in flight, and the products
   // start on the first chunks that arrive (vector loads return in the order they were issued).
@@ -366,7 +382,7 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   {
     const int first = c0 < c1 ? c0 : C - 1;
     load_chan(st, first);
-    load3(cur, first, c0 < c1);
+    load3_part(cur, first, c0 < c1, J0{}, JH{});
   }
 
   LnOut ln = ln_regs(xv, lg, lb, own, C, red);
@@ -393,6 +409,7 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   zero_pad<U8>(rx, nchunk, kPad);
   if constexpr (U8) publish_qsums(part, 3 * kQSums, qred);
   __syncthreads();
+  load3_part(cur, c0 < c1 ? c0 : C - 1, c0 < c1, JH{}, JN{});  // the rest of the first channel's rows
   float qt[3 * kQSums];
   if constexpr (U8) {
     const float tv = gather_qsums(3 * kQSums, qred);
@@ -609,9 +626,12 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       wh.nbytes[r] = have ? (int)row_bytes : 0;
     }
   };
-  // issue the loads of a located batch: its rows, then the per-row operands of its epilogue
-  auto request = [&](RowBatch<R, NCH, U8>& b, Meta& m, const Where& wh) {
-    b.load(wh.rows, wh.nbytes, lane);
+  // issue the loads of a located batch: its rows (chunks J0 .. J1-1), then the per-row operands of
+  // its epilogue
+  auto request_rows = [&](RowBatch<R, NCH, U8>& b, const Where& wh, auto j0, auto j1) {
+    b.template load<decltype(j0)::value, decltype(j1)::value>(wh.rows, wh.nbytes, lane);
+  };
+  auto request_ops = [&](Meta& m) {
     const int n = a.seg[m.seg].w.N;
     const int nl = m.loc0 + lane < n ? m.loc0 + lane : n - 1;
     m.ex = m.er = (h1)0.0f;
@@ -625,10 +645,14 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       m.qmx = a.seg[m.seg].w.mx[nl];
     }
   };
+  using J0 = std::integral_constant<int, 0>;
+  using JH = std::integral_constant<int, RowBatch<R, NCH, U8>::kHead>;
+  using JN = std::integral_constant<int, NCH>;
   auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int bi, bool live) {
     Where wh;
     locate(m, wh, bi, live);
-    request(b, m, wh);
+    request_rows(b, wh, J0{}, JN{});
+    request_ops(m);
   };
   auto consume = [&](const RowBatch<R, NCH, U8>& b, const Meta& m) {
     const Seg& sg = a.seg[m.seg];
@@ -700,9 +724,10 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     }
   }
 
-  // ---- first batch of rows ----
+  // ---- first batch of rows: the chunks that go out ahead of the prologue (see RowBatch::kHead) ----
   RowBatch<R, NCH, U8> A;
-  request(A, mA, whA);
+  request_rows(A, whA, J0{}, JH{});
+  request_ops(mA);
 
   // ---- prologue: stage the activation vector(s) in LDS ----
   {
@@ -756,6 +781,8 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     __syncthreads();
     if constexpr (U8) qtv = gather_qsums(a.nseg * kQSums, qred);
   }
+  // ---- the rest of the first batch ----
+  request_rows(A, whA, JH{}, JN{});
 
   if constexpr (!MULTI) {
     consume(A, mA);  // the host guarantees at most one batch per wave
