@@ -89,6 +89,7 @@ _SIGS = {
     "frhip_att_one_v5_1": (_i, [_i, _i] + [_vp] * 13 + [_WP] * 5 + [_vp] * 5),
     "frhip_att_one_v5": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 5),
     "frhip_argmax_f32": (_i, [_vp, _i, _vp, _vp]),
+    "frhip_argmax_blocks_f32": (_i, [_vp, _i, _vp, _i, _vp]),
     "frhip_gemm": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
     "frhip_copy_probe": (_i, [_vp, _vp, _sz, _vp]),
     "frhip_read_probe": (_i, [_vp, _sz, _vp, _vp]),

@@ -161,6 +161,56 @@ __global__ __launch_bounds__(512) void read_probe_kernel(const u32x4* __restrict
   if ((threadIdx.x & 63) == 0 && threadIdx.x == 0) sink[blockIdx.x] = v;
 }
 
+// The same over nblocks contiguous slices, one workgroup of 256 threads each: block b writes the
+// largest value of slice b and its (global) index, first occurrence on ties, as the pair
+// {float, int32} number b.  A slice is len elements (a multiple of 4; the last may be short or
+// empty: it reports -inf at index n).  The caller reduces the pairs (greater value, then smaller
+// index): with the logits in one slab that is 64 pairs instead of 65 536 values.
+__global__ __launch_bounds__(256) void argmax_blocks_f32_kernel(const float* __restrict__ x, int n, int len,
+                                                              float* pairs) {
+  __shared__ float bv[4];
+  __shared__ int bi[4];
+  const int lo = blockIdx.x * len;
+  const int hi = lo + len < n ? lo + len : n;
+  float best = -INFINITY;
+  int idx = n;
+  // thread t scans groups of 4 at lo + 4t, lo + 4t + 1024, ...: increasing indices, so '>' keeps the first
+  for (int i = lo + 4 * (int)threadIdx.x; i < hi; i += 1024) {
+    if (i + 4 <= hi) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (v.x > best) { best = v.x; idx = i; }
+      if (v.y > best) { best = v.y; idx = i + 1; }
+      if (v.z > best) { best = v.z; idx = i + 2; }
+      if (v.w > best) { best = v.w; idx = i + 3; }
+    } else {
+      for (int j = i; j < hi; j++)
+        if (x[j] > best) { best = x[j]; idx = j; }
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    float ov = __shfl_xor(best, off);
+    int oi = __shfl_xor(idx, off);
+    if (ov > best || (ov == best && oi < idx)) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    bv[threadIdx.x >> 6] = best;
+    bi[threadIdx.x >> 6] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; w++)
+      if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
+        best = bv[w];
+        idx = bi[w];
+      }
+    pairs[2 * blockIdx.x] = best;
+    reinterpret_cast<int32_t*>(pairs)[2 * blockIdx.x + 1] = idx;
+  }
+}
+
 // Index of the maximum, first occurrence on ties; single workgroup of 1024 threads.
 __global__ __launch_bounds__(1024) void argmax_f32_kernel(const float* __restrict__ x, int n, int32_t* out) {
   __shared__ float bv[16];
@@ -334,6 +384,16 @@ int frhip_read_probe(const void* src, size_t bytes, void* sink, frhip_stream s) 
   hipLaunchKernelGGL(read_probe_kernel, dim3(grid), dim3(512), 0, static_cast<hipStream_t>(s), (const u32x4*)src,
                      bytes / 16, (uint32_t*)sink);
   return check_launch("read_probe");
+}
+
+int frhip_argmax_blocks_f32(const float* x, int n, void* pairs, int nblocks, frhip_stream s) {
+  if (!x || !pairs) return set_error(FRHIP_EINVAL, "argmax: null pointer");
+  if (n <= 0 || nblocks <= 0) return set_error(FRHIP_ESHAPE, "argmax: empty input");
+  if (reinterpret_cast<uintptr_t>(x) % 16) return set_error(FRHIP_EINVAL, "argmax: x must be 16-byte aligned");
+  const int len = ((n + nblocks - 1) / nblocks + 3) / 4 * 4;
+  hipLaunchKernelGGL(argmax_blocks_f32_kernel, dim3(nblocks), dim3(256), 0, static_cast<hipStream_t>(s), x, n, len,
+                     static_cast<float*>(pairs));
+  return check_launch("argmax_blocks");
 }
 
 int frhip_argmax_f32(const float* logits, int n, int32_t* out_id, frhip_stream s) {

@@ -7,6 +7,7 @@
 #include <string>
 
 #include "kernels/hip/context.h"
+#include "kernels/hip/hip_model.h"
 #include "kernels/kernels.h"
 #include "model.h"
 #include "sampler.h"
@@ -185,7 +186,9 @@ long long fr_greedy_decode(void *m, int first_id, int steps, int *out_ids) {
     const auto t0 = std::chrono::steady_clock::now();
     for (int i = 0; i < steps; i++) {
       rwkv::Tensor out = model->Run(id);
-      id = argmax(out.data_ptr<float>(), static_cast<int>(out.numel()));
+      // the fused hip path has taken the argmax on the device (first index on ties, like argmax())
+      if (!rwkv::hip::device_argmax(model, out, &id))
+        id = argmax(out.data_ptr<float>(), static_cast<int>(out.numel()));
       out_ids[i] = id;
     }
     const auto t1 = std::chrono::steady_clock::now();

@@ -17,10 +17,13 @@ struct ModelExtra {
   Tensor emb_table;                 // [V, C]: one slab; Model::_embd_weights are row views into it
   std::vector<const void *> packed; // keys registered in the weight table, released with the model
   std::shared_ptr<DecodePlan> plan;
+  int32_t last_argmax = -1;               // index of the largest logit of the last fused one-token pass ...
+  const void *last_argmax_of = nullptr;   // ... and the logits buffer it belongs to
   ~ModelExtra();
 };
 
 std::shared_ptr<ModelExtra> extra_of(Model *model);
+bool device_argmax(Model *model, const Tensor &logits, int *id);
 
 // Defined in kernels/default/model_forward.cpp
 }  // namespace hip

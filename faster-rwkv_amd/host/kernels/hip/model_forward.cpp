@@ -14,6 +14,7 @@
 // FR_HIP_GENERIC=1 selects the operator-by-operator loop instead; FR_HIP_NO_GRAPH=1 keeps
 // the fused path but launches eagerly.
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 
 #include "kernels/hip/context.h"
@@ -27,6 +28,7 @@ namespace hip {
 
 struct DecodePlan {
   static constexpr int kRing = 64;
+  static constexpr int kArgmaxBlocks = 64;
   int L = 0, C = 0, F = 0, V = 0, n_logits = 0;
   Tensor x, ws, counter;
   Tensor logits_dev;
@@ -68,12 +70,13 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   p->counter = Tensor::Empty({1}, DType::kInt32, d);
   FRHIP_CHECK(frhip_fill(p->counter.data_ptr(), FRHIP_F32, 0.0f, 1, stream()));  // all-zero bits
   p->n_logits = static_cast<int>(model->_params.back().size(1));
-  p->logits_dev = Tensor::Empty({p->n_logits}, DType::kFloat32, d);
+  // behind the logits: kArgmaxBlocks {value, index} pairs of frhip_argmax_blocks_f32, copied to the host with them
+  p->logits_dev = Tensor::Empty({p->n_logits + 2 * DecodePlan::kArgmaxBlocks}, DType::kFloat32, d);
   void *h = nullptr;
   FRHIP_CHECK(frhip_host_malloc(&h, sizeof(int32_t) * DecodePlan::kRing));
   p->ring = static_cast<int32_t *>(h);
   for (auto &lh : p->logits_host) {
-    FRHIP_CHECK(frhip_host_malloc(&h, sizeof(float) * static_cast<size_t>(p->n_logits)));
+    FRHIP_CHECK(frhip_host_malloc(&h, sizeof(float) * (static_cast<size_t>(p->n_logits) + 2 * DecodePlan::kArgmaxBlocks)));
     lh = static_cast<float *>(h);
   }
   for (int l = 0; l < p->L; l++) {
@@ -191,8 +194,12 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
   RV_CHECK(hw != nullptr);
   FRHIP_CHECK(frhip_head(C, p.x.data_ptr(), P[pi].data_ptr(), P[pi + 1].data_ptr(), hw,
                          p.logits_dev.data_ptr<float>(), s));
-  FRHIP_CHECK(frhip_memcpy_async(p.logits_host[cur], p.logits_dev.data_ptr(), sizeof(float) * (size_t)p.n_logits,
-                                 FRHIP_D2H, s));
+  // The greedy sampler's step (Sampler::Sample with top_k = 1, sampler.cpp:28-32) on the device: a
+  // caller that only wants the most likely token need not read 4 * V bytes of fresh host memory.
+  FRHIP_CHECK(frhip_argmax_blocks_f32(p.logits_dev.data_ptr<float>(), p.n_logits,
+                                      p.logits_dev.data_ptr<float>() + p.n_logits, DecodePlan::kArgmaxBlocks, s));
+  FRHIP_CHECK(frhip_memcpy_async(p.logits_host[cur], p.logits_dev.data_ptr(),
+                                 sizeof(float) * ((size_t)p.n_logits + 2 * DecodePlan::kArgmaxBlocks), FRHIP_D2H, s));
 }
 
 Tensor ModelForward(Model *model, Device device, int id) {
@@ -237,7 +244,32 @@ Tensor ModelForward(Model *model, Device device, int id) {
   // is the step's one synchronisation point (the reference's is the blocking cudaMemcpy in
   // tensor.cpp:65-68).  The returned CPU tensor is a view, valid until the next-but-one call.
   FRHIP_CHECK(frhip_stream_sync(s));
+  {
+    // second step of the arg-max: greater value, then smaller index, over the per-slice pairs
+    const float *pairs = p.logits_host[cur] + p.n_logits;
+    float best = -INFINITY;
+    int32_t idx = p.n_logits;
+    for (int b = 0; b < DecodePlan::kArgmaxBlocks; b++) {
+      int32_t bi;
+      std::memcpy(&bi, pairs + 2 * b + 1, sizeof(bi));
+      if (pairs[2 * b] > best || (pairs[2 * b] == best && bi < idx)) {
+        best = pairs[2 * b];
+        idx = bi;
+      }
+    }
+    ex->last_argmax = idx < p.n_logits ? idx : 0;
+    ex->last_argmax_of = p.logits_host[cur];
+  }
   return Tensor::FromPtr(p.logits_host[cur], {p.n_logits}, DType::kFloat32, Device::kCPU);
+}
+
+// Index of the largest logit of the tensor `logits` if that tensor is the one the last one-token
+// forward pass of `model` returned and the pass computed the index on the device.
+bool device_argmax(Model *model, const Tensor &logits, int *id) {
+  auto ex = extra_of(model);
+  if (!ex || ex->last_argmax_of == nullptr || ex->last_argmax_of != logits.data_ptr()) return false;
+  *id = ex->last_argmax;
+  return true;
 }
 
 // Seq mode (reference: kernels/default/model_forward_seq.cpp:48-184): embedding rows are

@@ -232,6 +232,12 @@ int frhip_read_probe(const void *src, size_t bytes, void *sink, frhip_stream s);
 /* greedy sampler step (Sampler::Sample with top_k = 1, chat.cpp:76-77): index of the
  * largest logit, first one on ties, written to *out_id on the device. */
 int frhip_argmax_f32(const float *logits, int n, int32_t *out_id, frhip_stream s);
+/* The same in two steps, for a loop that copies the logits to the host anyway: the first step on the
+ * device over nblocks contiguous slices of x (16-byte aligned), writing nblocks pairs
+ * {fp32 largest value of the slice, int32 index of its first occurrence} to `pairs` (device, 8 * nblocks
+ * bytes; an empty slice reports -inf at index n); the second step, over the pairs (greater value,
+ * then smaller index), is the caller's. */
+int frhip_argmax_blocks_f32(const float *x, int n, void *pairs, int nblocks, frhip_stream s);
 
 #ifdef __cplusplus
 }

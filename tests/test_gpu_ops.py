@@ -173,6 +173,32 @@ def test_argmax_first_of_ties():
     assert out.numpy()[0] == 1234 == po.lib.orc_argmax(x.ctypes.data_as(C.c_void_p), 65536)
 
 
+@pytest.mark.parametrize("n,nblocks", [(65536, 64), (65529, 64), (1000, 64), (7, 3), (4096, 1)])
+def test_argmax_blocks_first_of_ties(n, nblocks):
+    """Per-slice {value, index} pairs, reduced as the host does (greater value, then smaller index),
+    give the oracle's arg-max: ragged lengths, slices that are short or empty, ties within a slice,
+    across slices and across the groups of four a thread scans."""
+    x = rng.standard_normal(n).astype(np.float32)
+    ties = sorted({n // 3, n // 3 + 1, n // 2, n - 1})
+    x[ties] = 9.0
+    pairs = DevBuf.empty(2 * nblocks, np.float32)
+    fr.check(L().frhip_argmax_blocks_f32(keep(x).ptr, n, pairs.ptr, nblocks, None))
+    raw = pairs.numpy()
+    vals, idxs = raw[0::2], raw[1::2].view(np.int32)
+    best, at = -np.inf, n
+    for v, i in zip(vals, idxs):
+        if v > best or (v == best and i < at):
+            best, at = v, int(i)
+    assert at == ties[0] == po.lib.orc_argmax(x.ctypes.data_as(C.c_void_p), n) and best == 9.0
+    ln = ((n + nblocks - 1) // nblocks + 3) // 4 * 4
+    for b in range(nblocks):  # every pair describes its own slice
+        sl = x[b * ln:min((b + 1) * ln, n)]
+        if len(sl):
+            assert vals[b] == sl.max() and idxs[b] == b * ln + int(np.argmax(sl))
+        else:
+            assert vals[b] == -np.inf and idxs[b] == n
+
+
 def test_gather_rows():
     tab = h(rng.standard_normal((1000, 256)))
     ids = np.array([5, 999, 0, 5, 123], np.int32)
