@@ -27,6 +27,97 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int BN = 128;
 constexpr int kGemmThreads = 256;
+// Fused epilogues, shared by the product kernels: acc[i][j] is the 32x32 block (i, j) of the wave's
+// (BM/2) x 64 tile at rows m0 + wm*(BM/2), columns n0 + wn*64; acc[i][j][v] is
+// C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the block.
+// FULL: the workgroup's tile lies inside the matrix, nothing is predicated.  (With a predicate per
+// element every store becomes a branch to an out-of-line block; on the 1024 x 6144 product that
+// was 11 of 59 us.)  The epilogue kind is uniform over the launch segment: one switch, and for the
+// kinds that read operands all 16 of a block are requested before the first is used.
+template <int BM, bool FULL>
+__device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg& sg, const f16v (&acc)[BM / 64][2],
+                                                int m0, int n0, int M, int N, int lane, int wm, int wn) {
+  constexpr int MI = BM / 64;
+  auto for_tile = [&](int i, int j, auto&& f) {
+    const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+      if constexpr (FULL)
+        f(v, true, (size_t)row * N + col);
+      else
+        f(v, row < M && col < N, (size_t)(row < M ? row : M - 1) * N + (col < N ? col : N - 1));
+    }
+  };
+  auto for_blocks = [&](auto&& g) {
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) g(i, j, acc[i][j]);
+  };
+  switch (sg.epi) {
+    case G_STORE_F16:
+      for_blocks([&](int i, int j, const f16v& c) {
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = (h1)c[v]; });
+      });
+      break;
+    case G_STORE_F32:
+      for_blocks([&](int i, int j, const f16v& c) {
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<float*>(sg.out)[o] = c[v]; });
+      });
+      break;
+    case G_SIGMOID:
+      for_blocks([&](int i, int j, const f16v& c) {
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = sigmoid_h((h1)c[v]); });
+      });
+      break;
+    case G_RELU2:
+      for_blocks([&](int i, int j, const f16v& c) {
+        for_tile(i, j, [&](int v, bool ok, size_t o) {
+          const h1 t = (h1)c[v];
+          if (ok) static_cast<h1*>(sg.out)[o] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
+        });
+      });
+      break;
+    case G_SILU:
+      for_blocks([&](int i, int j, const f16v& c) {
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = silu_h((h1)c[v]); });
+      });
+      break;
+    case G_RESIDUAL:
+      for_blocks([&](int i, int j, const f16v& c) {
+        h1 rx[16];
+        for_tile(i, j, [&](int v, bool, size_t o) { rx[v] = a.res_x[o]; });
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = rx[v] + (h1)c[v]; });
+      });
+      break;
+    case G_FFN_OUT:
+      for_blocks([&](int i, int j, const f16v& c) {
+        h1 rx[16], rr[16];
+        for_tile(i, j, [&](int v, bool, size_t o) {
+          rx[v] = a.res_x[o];
+          rr[v] = a.res_r[o];
+        });
+        for_tile(i, j, [&](int v, bool ok, size_t o) {
+          h1 r = __builtin_fmaf16((h1)c[v], rr[v], rx[v]);
+          if (a.div2) r = r / (h1)2.0f;
+          if (ok) static_cast<h1*>(sg.out)[o] = r;
+        });
+      });
+      break;
+    default: break;
+  }
+}
+
+template <int BM>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, const GemmSeg& sg, const f16v (&acc)[BM / 64][2], int m0,
+                                              int n0, int M, int N, int lane, int wm, int wn) {
+  if (m0 + BM <= M && n0 + BN <= N)
+    gemm_epilogue_t<BM, true>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+  else
+    gemm_epilogue_t<BM, false>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+}
+
 // BM = 128 (waves 2 x 2 of 64 x 64) or 64 (waves of 32 x 64), for launches that would otherwise
 // leave compute units idle.  BK = 64, or 128 for launches with about one workgroup per CU: with a
 // single wave per SIMD nothing hides the round trip of the next tile's loads, so a K step lasts
@@ -173,64 +264,142 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
     compute_tile();
   }
 
-  // epilogue: acc[i][j][v] is C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the 32x32 tile.
-  // The epilogue kind is uniform over the launch segment: branch once, and for the kinds that read
-  // operands request all 16 of a tile before the first is used.
-  auto for_tile = [&](int i, int j, auto&& f) {
-    const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+  gemm_epilogue<BM>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+}
+
+// ---------------------------------------------------------------------------
+// binary16 weights: four MFMA waves and a fifth that only moves data.
+//
+// A compute unit keeps about 64 KB of loads in flight, and a wave that asks for more stands at its
+// load instruction with everything behind it, MFMAs included.  In gemm_kernel the waves that
+// compute also load, so requests are outstanding only between "issue" and "store to LDS".  Here
+// wave 4 streams tiles global -> LDS directly (global_load_lds_dwordx4, no registers) into a ring
+// of kLdwStages K-steps of 64 and is the only wave that ever waits for memory: two steps (64 KB
+// for a 128 x 128 tile) are in flight all the time, and the MFMA waves meet it at one barrier
+// per step.  Same products in the same order as gemm_kernel: the results are bit-identical.
+//
+// LDS layout.  One load instruction brings 8 rows x 64 k = 8 x 128 contiguous bytes (fully
+// coalesced) and lands as 1 KB in lane order: lane l = row l/8, 16-byte slot l%8.  The lane asks
+// for k-segment (l%8) ^ (row%8), so k-segment q of row r sits in slot q ^ (r%8) and the MFMA
+// fragment reads (32 consecutive rows, one k-segment) spread over the banks without padding.
+// ---------------------------------------------------------------------------
+constexpr int kLdwThreads = 320;
+constexpr int kLdwStages = 4;
+constexpr int kLdwBK = 64;
+static constexpr size_t gemm_ldw_lds_bytes(int bm) { return (size_t)kLdwStages * (bm + BN) * kLdwBK * 2; }
+__device__ __forceinline__ int ldw_at(int row, int q) { return (row >> 3) * 1024 + (row & 7) * 128 + ((q ^ (row & 7)) * 16); }
+
+template <int BM>
+__global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
+  constexpr int MI = BM / 64;
+  constexpr int kABytes = BM * kLdwBK * 2, kBBytes = BN * kLdwBK * 2, kStageBytes = kABytes + kBBytes;
+  constexpr int kAInstr = kABytes / 1024, kBInstr = kBBytes / 1024, kPer = kAInstr + kBInstr;
+  static_assert(kPer == 32 || kPer == 24, "wait counts below are written for these");
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
+
+  int sidx = 0;
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-      const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-      f(v, row < M && col < N, (size_t)(row < M ? row : M - 1) * N + (col < N ? col : N - 1));
+  for (int i = 1; i < kGemmMaxSeg; i++) sidx += (i < a.nseg && (int)blockIdx.x >= a.tile_start[i]) ? 1 : 0;
+  const GemmSeg& sg = a.seg[sidx];
+  const int n0 = ((int)blockIdx.x - a.tile_start[sidx]) * BN;
+  const int m0 = blockIdx.y * BM;
+  const int M = a.M, K = a.K, N = sg.N;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nk = K / kLdwBK;
+
+  if (wave == 4) {
+    // ---- the loader ----
+    const int lr = lane >> 3, ls = (lane & 7) ^ lr;
+    // per-instruction row pointers; rows past M (N) repeat the last row and are never stored
+    const h1* pa[kAInstr];
+    const h1* pb[kBInstr];
+#pragma unroll
+    for (int b = 0; b < kAInstr; b++) {
+      int row = m0 + b * 8 + lr;
+      row = row < M ? row : M - 1;
+      pa[b] = sg.A + (size_t)row * K + ls * 8;
     }
-  };
 #pragma unroll
-  for (int i = 0; i < MI; i++) {
+    for (int b = 0; b < kBInstr; b++) {
+      int row = n0 + b * 8 + lr;
+      row = row < N ? row : N - 1;
+      pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + ls * 8;
+    }
+    auto issue = [&](int step) {
+      unsigned char* st = gemm_smem + (step % kLdwStages) * kStageBytes;
+      const int k0 = step * kLdwBK;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const f16v& c = acc[i][j];
-      switch (sg.epi) {
-        case G_STORE_F16:
-          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = (h1)c[v]; });
-          break;
-        case G_STORE_F32:
-          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<float*>(sg.out)[o] = c[v]; });
-          break;
-        case G_SIGMOID:
-          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = sigmoid_h((h1)c[v]); });
-          break;
-        case G_RELU2:
-          for_tile(i, j, [&](int v, bool ok, size_t o) {
-            const h1 t = (h1)c[v];
-            if (ok) static_cast<h1*>(sg.out)[o] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
-          });
-          break;
-        case G_SILU:
-          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = silu_h((h1)c[v]); });
-          break;
-        case G_RESIDUAL: {
-          h1 rx[16];
-          for_tile(i, j, [&](int v, bool, size_t o) { rx[v] = a.res_x[o]; });
-          for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = rx[v] + (h1)c[v]; });
-          break;
-        }
-        case G_FFN_OUT: {
-          h1 rx[16], rr[16];
-          for_tile(i, j, [&](int v, bool, size_t o) {
-            rx[v] = a.res_x[o];
-            rr[v] = a.res_r[o];
-          });
-          for_tile(i, j, [&](int v, bool ok, size_t o) {
-            h1 r = __builtin_fmaf16((h1)c[v], rr[v], rx[v]);
-            if (a.div2) r = r / (h1)2.0f;
-            if (ok) static_cast<h1*>(sg.out)[o] = r;
-          });
-          break;
-        }
-        default: break;
+      for (int b = 0; b < kAInstr; b++)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pa[b] + k0),
+                                         (__attribute__((address_space(3))) void*)(st + b * 1024), 16, 0, 0);
+#pragma unroll
+      for (int b = 0; b < kBInstr; b++)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pb[b] + k0),
+                                         (__attribute__((address_space(3))) void*)(st + kABytes + b * 1024), 16, 0, 0);
+    };
+    issue(0);
+    if (nk > 1) issue(1);
+    for (int k = 0; k < nk; k++) {
+      // step k has landed when at most the loads of step k+1 are outstanding (loads complete in order)
+      if (k + 1 < nk) {
+        if constexpr (kPer == 32)
+          __builtin_amdgcn_s_waitcnt(0x8F70);  // vmcnt(32)
+        else
+          __builtin_amdgcn_s_waitcnt(0x4F78);  // vmcnt(24)
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
       }
+      __builtin_amdgcn_s_barrier();            // barrier k: step k may be read, step k-1 has been read by all
+      if (k + 2 < nk) issue(k + 2);            // into the slot of step k-2
     }
+    return;
   }
+
+  // ---- the four MFMA waves: one barrier per step, matching the loader's ----
+  const int wm = wave >> 1, wn = wave & 1;
+  f16v acc[MI][2];
+#pragma unroll
+  for (int i = 0; i < MI; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+  for (int k = 0; k < nk; k++) {
+    __builtin_amdgcn_s_barrier();
+    const unsigned char* st = gemm_smem + (k % kLdwStages) * kStageBytes;
+    h8 fa[4][MI], fb[4][2];
+#pragma unroll
+    for (int kb = 0; kb < 4; kb++) {
+      const int q = kb * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < MI; i++)
+        fa[kb][i] = *reinterpret_cast<const h8*>(st + ldw_at(wm * (BM / 2) + i * 32 + (lane & 31), q));
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        fb[kb][j] = *reinterpret_cast<const h8*>(st + kABytes + ldw_at(wn * 64 + j * 32 + (lane & 31), q));
+    }
+#pragma unroll
+    for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+      for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kb][i], fb[kb][j], acc[i][j], 0, 0, 0);
+  }
+  gemm_epilogue<BM>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+}
+
+template <int BM>
+static void gemm_ldw_launch(dim3 grid, hipStream_t st, const GemmArgs& a) {
+  constexpr size_t lds = gemm_ldw_lds_bytes(BM);
+  static bool raised = false;
+  if (!raised) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_ldw_kernel<BM>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL((gemm_ldw_kernel<BM>), grid, dim3(kLdwThreads), lds, st, a);
 }
 
 static constexpr size_t gemm_lds_bytes(int bm, int bk) { return (size_t)(bm + BN) * (bk + 8) * 2; }
@@ -279,6 +448,16 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what) {
   static const int force_bk = env_bk();
   const bool deep = force_bk ? force_bk == 128 : true;
   const bool deep_ok = deep && a.K % 128 == 0;
+  // binary16 weights go to the kernel with the loader wave (FRHIP_GEMM_LDW=0 selects the other one:
+  // measurement aid); uint8 weights need the registers in between for the dequantisation
+  static const bool ldw = !(getenv("FRHIP_GEMM_LDW") && atoi(getenv("FRHIP_GEMM_LDW")) == 0);
+  if (!u8 && ldw) {
+    if (small)
+      gemm_ldw_launch<64>(dim3(tiles, (a.M + 63) / 64), st, a);
+    else
+      gemm_ldw_launch<128>(dim3(tiles, m128), st, a);
+    return check_launch(what);
+  }
   if (small) {
     dim3 grid(tiles, (a.M + 63) / 64);
     if (deep_ok) FR_GEMM_LAUNCH(64, 128); else FR_GEMM_LAUNCH(64, 64);
