@@ -4,14 +4,17 @@
 //
 // Both operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
 // a lane's A (or B) fragment is 8 consecutive k of one row, i.e. one 16-byte load.
-// Workgroup tile 128x128 (64x128 for launches that would otherwise leave CUs idle), K step 64 (128 for
-// launches of about one workgroup per CU),
-// 256 threads = 2x2 waves of 64x64 (2x2 MFMA tiles, 64 fp32 accumulators per lane).  Tiles of X and Wt go global -> registers -> LDS
-// (rows padded by 16 bytes against bank conflicts); the loads of step k+1 are issued
-// before the MFMAs of step k.  uint8 weights are dequantised to binary16 on their way
-// into LDS with the same formula as the one-token kernels, so the product sees exactly
-// the dequantised matrix.  Products are exact in fp32, accumulation is fp32, and the
-// result is rounded once to the output type (kernels/cuda/matmul.cpp:38-42,64-68).
+// Workgroup tile 128x128 (64x128 for launches that would otherwise leave CUs idle), 2x2 compute
+// waves of 64x64 (2x2 MFMA tiles, 64 fp32 accumulators per lane).  Two kernels:
+//   gemm_ldw_kernel  binary16 weights: a fifth wave streams the tiles global -> LDS directly
+//                    through a ring of four 64-deep K steps; the compute waves never load;
+//   gemm_kernel      uint8 weights: tiles go global -> registers -> LDS (rows padded by 16 bytes
+//                    against bank conflicts), the loads of step k+1 issued before the MFMAs of
+//                    step k, and are dequantised to binary16 on the way into LDS with the same
+//                    formula as the standalone dequantisation, so the product sees exactly the
+//                    dequantised matrix.
+// Products are exact in fp32, accumulation is fp32 in ascending k, and the result is rounded once
+// to the output type (kernels/cuda/matmul.cpp:38-42,64-68); both kernels give the same bits.
 // Independent products over the same T and K share one launch ("segments"), each with
 // its own X, W and fused epilogue.
 #include <climits>
