@@ -292,7 +292,7 @@ def main():
     # HBM bytes per launch (average over the launches of one token) from the FETCH_SIZE / WRITE_SIZE
     # hardware counters, scaled by a copy kernel of known size: measured with rocprofv3 --pmc on this
     # command and kept in profiles/decode_rwkv4_1b5_fp16_hbm_traffic.md; not measured for uint8.
-    traffic = round((2914.5e6 + 2.3e6) / n_launch) if args.dtype == "fp16" else None
+    traffic = round((2915.2e6 + 2.3e6) / n_launch) if args.dtype == "fp16" else None
     out = {
         "metric": "decode tok/s (RWKV-4 1.5B-shaped, bs1, greedy)", "value": round(tok_s, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
