@@ -469,12 +469,13 @@ static int launch_ln_mix(int T, int C, const void* x, const void* state, const v
 }
 
 // chunk length for a scan of T steps when one chunk occupies `units` workgroup-sized units:
-// enough chunks to fill the device (~4 units per CU), chunks of at least 8 steps
+// enough chunks to fill the device (~4 units per CU), chunks of at least 16 steps (the serial pass
+// over the chunks costs about 0.18 us per chunk: at T = 1024, 64 chunks of 16 beat 128 of 8)
 static int pick_chunk(int T, int units) {
   int want = (4 * compute_units() + units - 1) / units;
   if (want < 1) want = 1;
   int Lc = (T + want - 1) / want;
-  if (Lc < 8) Lc = 8;
+  if (Lc < 16) Lc = 16;
   if (Lc > 64) Lc = 64;
   return Lc;
 }
