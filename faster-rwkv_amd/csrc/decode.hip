@@ -162,7 +162,11 @@ struct RowBatch {
   // 16 loads put about 8 of them first, then the prologue, then the rest; for smaller ones holding
   // loads back only idles the memory (measured: 24 loads, 6 first: 9.60 -> 9.33 us; 16 loads, 8
   // first: 7.11 -> 7.32 us; 12 loads, 6 first: 6.81 -> 7.12 us).
-  static constexpr int kHead = R * NCH <= 16 ? NCH : (8 / R < 1 ? 1 : 8 / R);
+  // uint8 rows cost two VALU operations per code, about as long as their bytes take to arrive: the
+  // sooner the prologue's barrier, the more of the products run under the stream, so only about
+  // six loads go first there.
+  static constexpr int kFirst = U8 ? 6 : 8;
+  static constexpr int kHead = R * NCH <= (U8 ? 6 : 16) ? NCH : (kFirst / R < 1 ? 1 : kFirst / R);
 
   // All rows against one staged vector, each chunk of which is read from LDS once.  Binary16 rows:
   // acc[r] = sum_k w[k] x[k] against a binary16 vector; uint8 rows: acc[r] = sum_k q[k] xr[k]
@@ -646,7 +650,8 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     }
   };
   using J0 = std::integral_constant<int, 0>;
-  using JH = std::integral_constant<int, RowBatch<R, NCH, U8>::kHead>;
+  // (a wave with several batches streams anyway: its first batch goes out whole)
+  using JH = std::integral_constant<int, MULTI ? NCH : RowBatch<R, NCH, U8>::kHead>;
   using JN = std::integral_constant<int, NCH>;
   auto fetch = [&](RowBatch<R, NCH, U8>& b, Meta& m, int bi, bool live) {
     Where wh;
