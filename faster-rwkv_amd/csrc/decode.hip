@@ -340,7 +340,8 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
     b.r.template load<decltype(j0)::value, decltype(j1)::value>(rr, nb, lane);
   };
   using J0 = std::integral_constant<int, 0>;
-  using JH = std::integral_constant<int, RowBatch<3, NCH, U8>::kHead>;  // requested ahead of the prologue
+  // requested ahead of the prologue: uint8, one chunk of each row (its products take as long as its bytes)
+  using JH = std::integral_constant<int, U8 ? 1 : RowBatch<3, NCH, U8>::kHead>;
   using JN = std::integral_constant<int, NCH>;
   auto load3 = [&](Rows3& b, int n, bool live) { load3_part(b, n, live, J0{}, JN{}); };
   // Every global operand is requested before the first wait, operands of the prologue first: the
