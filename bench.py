@@ -300,7 +300,7 @@ def main():
         "dtype": "f16" if args.dtype == "fp16" else "u8 weights, f16 activations, f32 accumulate",
         "data": "synthetic (random-init weights, greedy token ids)",
         "config": {"workload": cfg["workload"], "strategy": cfg["strategy"], "steps": args.steps,
-                   "host_loop": "Model::Run (logits and 64 per-slice arg-max pairs to pinned host memory) + host reduction of the pairs per token"},
+                   "host_loop": "Model::Run (the head stores logits and 64 per-slice arg-max pairs to pinned host memory) + host reduction of the pairs per token"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "row-streaming matrix-vector kernels (att_front/att_out/ffn_front/ffn_out/head), "

@@ -86,6 +86,7 @@ _SIGS = {
     "frhip_att_one_v4": (_i, [_i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),
     "frhip_ffn_one": (_i, [_i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
     "frhip_head": (_i, [_i, _vp, _vp, _vp, _WP, _vp, _vp]),
+    "frhip_head_mirror": (_i, [_i, _vp, _vp, _vp, _WP, _vp, _vp, _vp]),
     "frhip_att_one_v5_1": (_i, [_i, _i] + [_vp] * 13 + [_WP] * 5 + [_vp] * 5),
     "frhip_att_one_v5": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 5),
     "frhip_argmax_f32": (_i, [_vp, _i, _vp, _vp]),

@@ -539,6 +539,7 @@ struct RowsArgs {
   const h1* res_x;  // E_RESIDUAL, E_FFN_OUT
   const h1* res_r;  // E_FFN_OUT
   int res_n;        // elements of res_x / res_r that may be read (1 when no epilogue uses them)
+  float* mirror;    // E_LOGITS: second destination of every value (memory the host reads), or null
   int div2;
 };
 
@@ -559,7 +560,12 @@ __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, i
       static_cast<h1*>(sg.out)[n] = o;
       break;
     }
-    case E_LOGITS: static_cast<float*>(sg.out)[n] = (float)(h1)sum; break;
+    case E_LOGITS: {
+      const float v = (float)(h1)sum;
+      static_cast<float*>(sg.out)[n] = v;
+      if (a.mirror) a.mirror[n] = v;
+      break;
+    }
     case E_SILU: static_cast<h1*>(sg.out)[n] = silu_h((h1)sum); break;
     default: break;
   }
@@ -1339,6 +1345,11 @@ extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const 
 
 extern "C" int frhip_head(int C, const void* x, const void* ln_w, const void* ln_b, const frhip_weight* head,
                           float* logits, frhip_stream s) {
+  return frhip_head_mirror(C, x, ln_w, ln_b, head, logits, nullptr, s);
+}
+
+extern "C" int frhip_head_mirror(int C, const void* x, const void* ln_w, const void* ln_b, const frhip_weight* head,
+                                 float* logits, float* mirror, frhip_stream s) {
   FR_TRY(check_embd(C));
   FR_TRY(check_vec(x, "x is null or misaligned"));
   FR_TRY(check_vec(ln_w, "ln_w is null or misaligned"));
@@ -1349,6 +1360,7 @@ extern "C" int frhip_head(int C, const void* x, const void* ln_w, const void* ln
   a.prologue = P_LN;
   a.nvec = 1;
   a.x = (const h1*)x; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+  a.mirror = mirror;
   add_seg(a, head, 0, E_LOGITS, logits);
   return launch_rows(a, head->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "head");
 }

@@ -6,8 +6,8 @@
 // captured once into a HIP graph and replayed.  The token-shift states ping-pong between
 // two buffers (the kernel that writes the new state runs while other workgroups still read
 // the old one), hence one graph per parity.  The token id reaches the first kernel through a
-// small ring in pinned host memory, and the graph's last node copies the logits to pinned host
-// memory, so a step costs the host one graph launch and one stream wait.  The recurrent state that model code sees
+// small ring in pinned host memory, and the head kernel stores the logits to pinned host memory as
+// well as to device memory, so a step costs the host one graph launch and one stream wait.  The recurrent state that model code sees
 // (Model::states()) is kept as views of these buffers; states assigned from outside
 // (ResetStates, LoadStateFile, set_states) are copied in on the next call.
 //
@@ -32,7 +32,7 @@ struct DecodePlan {
   int L = 0, C = 0, F = 0, V = 0, n_logits = 0;
   Tensor x, ws, counter;
   Tensor logits_dev;
-  float *logits_host[2] = {nullptr, nullptr};  // pinned; the graph's last node copies into it
+  float *logits_host[2] = {nullptr, nullptr};  // pinned; the head kernel stores the logits here too, the arg-max pairs follow
   int32_t *ring = nullptr;                     // pinned; token ids, read by the first kernel
   uint32_t fed = 0;                            // tokens fed so far == the device counter
   bool v5 = false;                      // RWKV-5.x: state is (shift, [H,S,S] matrix, shift)
@@ -70,8 +70,7 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   p->counter = Tensor::Empty({1}, DType::kInt32, d);
   FRHIP_CHECK(frhip_fill(p->counter.data_ptr(), FRHIP_F32, 0.0f, 1, stream()));  // all-zero bits
   p->n_logits = static_cast<int>(model->_params.back().size(1));
-  // behind the logits: kArgmaxBlocks {value, index} pairs of frhip_argmax_blocks_f32, copied to the host with them
-  p->logits_dev = Tensor::Empty({p->n_logits + 2 * DecodePlan::kArgmaxBlocks}, DType::kFloat32, d);
+  p->logits_dev = Tensor::Empty({p->n_logits}, DType::kFloat32, d);
   void *h = nullptr;
   FRHIP_CHECK(frhip_host_malloc(&h, sizeof(int32_t) * DecodePlan::kRing));
   p->ring = static_cast<int32_t *>(h);
@@ -192,14 +191,14 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
   }
   const frhip_weight *hw = find_weight(P[pi + 2]);
   RV_CHECK(hw != nullptr);
-  FRHIP_CHECK(frhip_head(C, p.x.data_ptr(), P[pi].data_ptr(), P[pi + 1].data_ptr(), hw,
-                         p.logits_dev.data_ptr<float>(), s));
-  // The greedy sampler's step (Sampler::Sample with top_k = 1, sampler.cpp:28-32) on the device: a
-  // caller that only wants the most likely token need not read 4 * V bytes of fresh host memory.
-  FRHIP_CHECK(frhip_argmax_blocks_f32(p.logits_dev.data_ptr<float>(), p.n_logits,
-                                      p.logits_dev.data_ptr<float>() + p.n_logits, DecodePlan::kArgmaxBlocks, s));
-  FRHIP_CHECK(frhip_memcpy_async(p.logits_host[cur], p.logits_dev.data_ptr(),
-                                 sizeof(float) * ((size_t)p.n_logits + 2 * DecodePlan::kArgmaxBlocks), FRHIP_D2H, s));
+  // The head stores every logit twice: to device memory, where the greedy sampler's step (Sampler::Sample
+  // with top_k = 1, sampler.cpp:28-32) reads them, and to the pinned host buffer the call returns, so that
+  // they cross the bus while the product runs; the per-slice pairs of the arg-max go to the host directly.
+  // A caller that only wants the most likely token need not read 4 * V bytes of fresh host memory.
+  FRHIP_CHECK(frhip_head_mirror(C, p.x.data_ptr(), P[pi].data_ptr(), P[pi + 1].data_ptr(), hw,
+                                p.logits_dev.data_ptr<float>(), p.logits_host[cur], s));
+  FRHIP_CHECK(frhip_argmax_blocks_f32(p.logits_dev.data_ptr<float>(), p.n_logits, p.logits_host[cur] + p.n_logits,
+                                      DecodePlan::kArgmaxBlocks, s));
 }
 
 Tensor ModelForward(Model *model, Device device, int id) {
@@ -240,7 +239,7 @@ Tensor ModelForward(Model *model, Device device, int id) {
     st[l][0] = p.views[p.parity][l][0];
     st[l][last] = p.views[p.parity][l][last];
   }
-  // The graph's last node has copied the logits into pinned host memory; waiting for the stream
+  // The head kernel has stored the logits into pinned host memory; waiting for the stream
   // is the step's one synchronisation point (the reference's is the blocking cudaMemcpy in
   // tensor.cpp:65-68).  The returned CPU tensor is a view, valid until the next-but-one call.
   FRHIP_CHECK(frhip_stream_sync(s));

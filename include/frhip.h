@@ -149,6 +149,11 @@ int frhip_ffn_one(int C, int F, const void *x, const void *sx, const void *ln_w,
 
 /* layernorm(ln_out) -> head matmul -> cast to fp32: kernels/default/model_forward.cpp:180-188. */
 int frhip_head(int C, const void *x, const void *ln_w, const void *ln_b, const frhip_weight *head, float *logits, frhip_stream s);
+/* The same with a second destination: every logit is also stored to mirror [N] (fp32), meant for pinned host
+ * memory, so that the values cross the bus while the product runs instead of in a copy after it (the reference
+ * copies after: tensor.cpp:65-68).  mirror may be null. */
+int frhip_head_mirror(int C, const void *x, const void *ln_w, const void *ln_b, const frhip_weight *head, float *logits,
+                      float *mirror, frhip_stream s);
 
 /* att_one_v5_1 (RWKV-5.1/5.2, one token): kernels/cuda/att.cu:267-335,393-425.
  * s [H][S][S] fp32 ([head][key][value]); t_decay, t_first [H][S]; lx_w, lx_b [C] fp32.

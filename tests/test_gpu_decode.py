@@ -1,4 +1,5 @@
 """GPU parity tests of the fused one-token operators and of whole-model greedy decode."""
+import ctypes as C
 import numpy as np
 import pytest
 
@@ -199,6 +200,28 @@ def test_head(quant):
         assert np.abs(got - ref).max() <= 4e-3
     else:
         assert_close_f16(got.astype(np.float16), ref.astype(np.float16), max_ulp=2, max_frac=0.05, what="logits")
+
+
+def test_head_mirror_in_pinned_host_memory():
+    """frhip_head_mirror stores every logit to a second buffer as well; with that buffer in pinned host
+    memory the host reads, after a stream wait, exactly what the device buffer holds."""
+    C_, V_ = 2048, 8192
+    x, ln_w, ln_b = h(rng.standard_normal(C_) * 3), h(1 + 0.1 * rng.standard_normal(C_)), h(0.1 * rng.standard_normal(C_))
+    hw, _ = make_weight(h(rng.standard_normal((C_, V_)) * 0.02), False)
+    out = DevBuf.empty(V_, np.float32)
+    hp = C.c_void_p()
+    fr.check(L().frhip_host_malloc(C.byref(hp), 4 * V_))
+    try:
+        host = np.ctypeslib.as_array(C.cast(hp, C.POINTER(C.c_float)), shape=(V_,))
+        host[:] = -1.0
+        fr.check(L().frhip_head_mirror(C_, keep(x).ptr, keep(ln_w).ptr, keep(ln_b).ptr, hw.ref, out.ptr, hp, None))
+        fr.check(L().frhip_device_sync())
+        assert np.array_equal(host, out.numpy())
+        ref = DevBuf.empty(V_, np.float32)
+        fr.check(L().frhip_head(C_, keep(x).ptr, keep(ln_w).ptr, keep(ln_b).ptr, hw.ref, ref.ptr, None))
+        assert np.array_equal(ref.numpy(), out.numpy())
+    finally:
+        fr.check(L().frhip_host_free(hp))
 
 
 def _greedy_pair(L_, C_, F_, V_, quant, steps, seed):
