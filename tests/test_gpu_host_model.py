@@ -259,3 +259,32 @@ def test_sampled_generation_follows_the_oracle_sampler(model_files):
         tok = so.sample(m.run(tok), 1.2, 50, 0.9, g)
         assert tok == int(toks[i]), i
     m.close()
+
+
+# ---------------------------------------------------------------------------
+# committed golden vectors (tests/golden/oracle_small_models.npz): the HIP path on the same
+# synthetic models, one-token steps and seq mode, within the stated tolerance of the fixture
+# ---------------------------------------------------------------------------
+import sys as _sys
+
+_sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+import make_oracle_golden as _mg
+
+_GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "oracle_small_models.npz"))
+
+
+@pytest.mark.parametrize("name", sorted(_mg.CASES))
+def test_hip_model_against_committed_golden_logits(name, tmp_path):
+    version, L, C, F, V, H, seed, quant = _mg.CASES[name]
+    params, emb = make_model(version, L, C, F, V, H, seed=seed)
+    path = str(tmp_path / (name + ".fr"))
+    fr.write_fr(path, {4: "4", 50: "5", 52: "5.2"}[version], L, C, F, H, params, emb)
+    m = fr.Model(path, "hip int8" if quant else "hip fp16")
+    gold_one, gold_seq = _GOLD[name + "_one"], _GOLD[name + "_seq_last"]
+    for i, t in enumerate(_GOLD["tokens"]):
+        lh = m.run(int(t))
+        assert np.abs(lh - gold_one[i]).max() <= 2e-2, (name, i)
+        assert _same_token(lh, gold_one[i])
+    m.reset()
+    ls = m.run([int(t) for t in _GOLD["tokens"]])
+    assert np.abs(ls - gold_seq).max() <= 2e-2 and _same_token(ls, gold_seq)
