@@ -35,7 +35,14 @@ struct GemmArgs {
   int div2;
 };
 
-int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what);
+// dq: optional scratch of gemm_dequant_bytes(a) bytes.  With it, uint8 weights of a launch with at least
+// kDequantRows rows are expanded once to binary16 (the standalone dequantisation: the same bits as the
+// in-kernel one) and the launch takes the binary16 kernel.
+int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq = nullptr);
+constexpr int kDequantRows = 192;
+// uint8 [N][K] -> binary16 [N][K] with the frozen formula (ops.hip)
+int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,
+                     hipStream_t st);
 void gemm_add_seg(GemmArgs& a, const void* A, const frhip_weight* w, void* out, int epi);
 
 }  // namespace frhip

@@ -434,9 +434,22 @@ static int env_bk() {
   return e ? atoi(e) : 0;
 }
 
-int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what) {
+int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq) {
   if (a.M <= 0) return 0;
   if (a.K <= 0 || a.K % 64 != 0) return set_error(FRHIP_ESHAPE, "gemm: K must be a positive multiple of 64");
+  if (u8 && dq && a.M >= kDequantRows) {
+    // Expanding N x K codes costs 3 bytes of traffic per weight; the uint8 kernel's in-flight dequantisation
+    // costs the launch about 0.4 x 2 T FLOP per weight at the binary16 kernel's rate: from a few hundred rows
+    // on, one expansion and the binary16 kernel win.
+    h1* dst = static_cast<h1*>(dq);
+    for (int s = 0; s < a.nseg; s++) {
+      GemmSeg& g = a.seg[s];
+      if (int rc = dequant_u8_async(g.B, g.mx, g.rx, g.my, g.ry, dst, a.K, g.N, st)) return rc;
+      g.B = reinterpret_cast<const unsigned char*>(dst);
+      dst += (size_t)g.N * a.K;
+    }
+    u8 = false;
+  }
   int tiles = 0;
   for (int s = 0; s < a.nseg; s++) {
     a.tile_start[s] = tiles;

@@ -3,6 +3,7 @@
 // scalar_div_, vgather), weight preparation, and the greedy sampler's argmax.
 #include "device_utils.h"
 #include "frhip_internal.h"
+#include "gemm.h"
 
 #pragma clang fp contract(off)
 
@@ -247,6 +248,14 @@ __global__ __launch_bounds__(1024) void argmax_f32_kernel(const float* __restric
   }
 }
 
+int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,
+                     hipStream_t st) {
+  const size_t words = (size_t)N * (K / 4);
+  hipLaunchKernelGGL(dequant_u8_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, (const uint32_t*)q, mx, rx, my, ry,
+                     (h4*)dst, K, N);
+  return check_launch("dequant_u8");
+}
+
 }  // namespace frhip
 
 using namespace frhip;
@@ -359,11 +368,8 @@ int frhip_dequant_u8(const frhip_weight* w, void* dst, frhip_stream s) {
   if (!w || !w->data || !dst) return set_error(FRHIP_EINVAL, "dequant: null pointer");
   if (w->dtype != FRHIP_U8 || !w->mx || !w->rx || !w->my || !w->ry) return set_error(FRHIP_EINVAL, "dequant: not a uint8 weight");
   if (w->K <= 0 || w->N <= 0 || w->K % 4 != 0) return set_error(FRHIP_ESHAPE, "dequant: K must be a multiple of 4");
-  const size_t words = (size_t)w->N * (w->K / 4);
-  hipLaunchKernelGGL(dequant_u8_kernel, dim3(blocks_for(words, 256)), dim3(256), 0, static_cast<hipStream_t>(s),
-                     (const uint32_t*)w->data, (const h1*)w->mx, (const h1*)w->rx, (const h1*)w->my, (const h1*)w->ry,
-                     (h4*)dst, w->K, w->N);
-  return check_launch("dequant_u8");
+  return dequant_u8_async((const unsigned char*)w->data, (const h1*)w->mx, (const h1*)w->rx, (const h1*)w->my,
+                          (const h1*)w->ry, (h1*)dst, w->K, w->N, static_cast<hipStream_t>(s));
 }
 
 int frhip_copy_probe(void* dst, const void* src, size_t bytes, frhip_stream s) {

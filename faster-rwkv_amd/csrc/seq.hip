@@ -484,6 +484,12 @@ static int pick_chunk(int T, int units) {
 
 using namespace frhip;
 
+static size_t seq_dequant_bytes(int C, int F) {
+  const size_t cc = (size_t)C * C, cf = (size_t)C * F;
+  const size_t att = 4 * cc, ffn = cc + cf;
+  return 2 * (att > ffn ? att : ffn);
+}
+
 extern "C" size_t frhip_seq_workspace_bytes(int T, int C, int F) {
   if (T <= 0 || C <= 0 || F <= 0) return 0;
   const size_t tc = (size_t)T * C;
@@ -492,6 +498,8 @@ extern "C" size_t frhip_seq_workspace_bytes(int T, int C, int F) {
   // scan scratch: RWKV-4 6 x [nchunk][C] fp32 with nchunk <= T/8+1; RWKV-5 2 x [nchunk][C*64] fp32
   const size_t nchunk = (size_t)T / 8 + 1;
   n += 6 * al256(4 * nchunk * C) + 2 * al256(4 * nchunk * (size_t)C * 64);
+  // binary16 expansion of the uint8 weights of one launch: the largest group is k,v,r,g or ffn r,k
+  n += al256(seq_dequant_bytes(C, F));
   return n;
 }
 
@@ -500,6 +508,7 @@ struct SeqWs {
   h1 *m0, *m1, *m2, *m3, *g, *gated, *vx;
   float *f0, *f1, *f2, *f3;
   float* scan;
+  h1* dq;  // binary16 expansion of one launch's uint8 weights
 };
 SeqWs carve_seq(void* ws, int T, int C, int F) {
   const size_t tc = (size_t)T * C;
@@ -518,6 +527,9 @@ SeqWs carve_seq(void* ws, int T, int C, int F) {
   w.vx = reinterpret_cast<h1*>(p);
   p += al256(2 * (size_t)T * F);
   w.scan = reinterpret_cast<float*>(p);
+  const size_t nchunk = (size_t)T / 8 + 1;
+  p += 6 * al256(4 * nchunk * C) + 2 * al256(4 * nchunk * (size_t)C * 64);
+  w.dq = reinterpret_cast<h1*>(p);
   return w;
 }
 }  // namespace
@@ -545,13 +557,13 @@ extern "C" int frhip_ffn_seq(int T, int C, int F, const void* x, const void* sx,
   gemm_add_seg(a, w.m1, rw, w.m2, G_SIGMOID);  // r
   gemm_add_seg(a, w.m0, kw, w.vx, G_RELU2);    // vx
   if (kw->dtype != rw->dtype) return set_error(FRHIP_EINVAL, "ffn_seq: key/receptance dtypes differ");
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "ffn_seq r,k"));
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "ffn_seq r,k", w.dq));
   GemmArgs b;
   memset(&b, 0, sizeof(b));
   b.M = T; b.K = F;
   b.res_x = (const h1*)x; b.res_r = w.m2; b.div2 = post_div2 ? 1 : 0;
   gemm_add_seg(b, w.vx, vw, x_out, G_FFN_OUT);
-  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v");
+  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v", w.dq);
 }
 
 // RWKV-4 sequence attention.  The reference has no such operator
@@ -584,7 +596,7 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   gemm_add_seg(a, w.m0, kw, w.f0, G_STORE_F32);  // k
   gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
   gemm_add_seg(a, w.m2, rw, w.m3, G_SIGMOID);    // r
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v4 k,v,r"));
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v4 k,v,r", w.dq));
 
   Wkv4Seq q;
   q.T = T; q.C = C;
@@ -606,7 +618,7 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   b.M = T; b.K = C;
   b.res_x = (const h1*)x;
   gemm_add_seg(b, w.m3, ow, x_out, G_RESIDUAL);
-  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v4 out");
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v4 out", w.dq);
 }
 
 // Shared by RWKV-5.0 (no gate, u and w per head) and RWKV-5.2.
@@ -641,7 +653,7 @@ static int att_seq_v5_impl(bool v50, int T, int C, int H, const void* x, const v
   gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
   gemm_add_seg(a, w.m2, rw, w.f2, G_STORE_F32);  // r
   if (!v50) gemm_add_seg(a, w.m3, gw, w.g, G_SILU);  // g
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5 k,v,r,g"));
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5 k,v,r,g", w.dq));
 
   Wkv5Seq q;
   q.T = T; q.C = C; q.H = H;
@@ -664,7 +676,7 @@ static int att_seq_v5_impl(bool v50, int T, int C, int H, const void* x, const v
   b.M = T; b.K = C;
   b.res_x = (const h1*)x;
   gemm_add_seg(b, w.gated, ow, x_out, G_RESIDUAL);
-  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5 out");
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5 out", w.dq);
 }
 
 // att_seq_v5_2 (kernels/cuda/att_seq.cu:368-423,464-493).
