@@ -92,6 +92,7 @@ _SIGS = {
     "frhip_argmax_f32": (_i, [_vp, _i, _vp, _vp]),
     "frhip_argmax_blocks_f32": (_i, [_vp, _i, _vp, _i, _vp]),
     "frhip_gemm": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
+    "frhip_gemm_act": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
     "frhip_copy_probe": (_i, [_vp, _vp, _sz, _vp]),
     "frhip_read_probe": (_i, [_vp, _sz, _vp, _vp]),
     "frhip_seq_workspace_bytes": (_sz, [_i, _i, _i]),

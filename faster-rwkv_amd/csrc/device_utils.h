@@ -82,14 +82,22 @@ __device__ __forceinline__ h1 mix1(h1 xx, h1 sx, h1 m) { return (xx * m) + (sx *
 // formed in fp32 (a few units in the last place of error); only when that lies so close to the
 // midpoint of two binary16 values that the error could change the rounding, or in the binary16
 // subnormal range, is the double path taken.  The result is the double path's bit for bit.
-__device__ __forceinline__ h1 sigmoid_h(h1 x) {
+__device__ __forceinline__ h1 sigmoid_h_exact(h1 x) {
+  const double s = 1.0 / (1.0 + exp(-(double)(float)x));
+  return (h1)(float)s;
+}
+// The fp32 value rounded to binary16; *safe says whether that is certainly sigmoid_h_exact's result.
+__device__ __forceinline__ h1 sigmoid_h_fast(h1 x, bool* safe) {
   const float xf = (float)x;
   const float s32 = 1.0f / (1.0f + expf(-xf));
   const uint32_t frac = __float_as_uint(s32) & 0x1FFFu;  // the 13 fp32 mantissa bits binary16 drops
-  const bool safe = s32 > 1e-4f && (frac < 0x1000u - 64u || frac > 0x1000u + 64u);
-  if (safe) return (h1)s32;
-  double s = 1.0 / (1.0 + exp(-(double)xf));
-  return (h1)(float)s;
+  *safe = s32 > 1e-4f && (frac < 0x1000u - 64u || frac > 0x1000u + 64u);
+  return (h1)s32;
+}
+__device__ __forceinline__ h1 sigmoid_h(h1 x) {
+  bool safe;
+  const h1 y = sigmoid_h_fast(x, &safe);
+  return safe ? y : sigmoid_h_exact(x);
 }
 
 // kernels/cuda/att.cu:145-152

@@ -29,6 +29,8 @@ struct GemmSeg {
 struct GemmArgs {
   int M, K, nseg;
   int tile_start[kGemmMaxSeg + 1];  // first N-tile of each segment
+  // gemm_vw_kernel: a segment's tiles are vw_base (the first vw_wide of them vw_base + 1) blocks of 32 columns wide
+  int vw_base[kGemmMaxSeg], vw_wide[kGemmMaxSeg], vw_maxw, vw_ns;
   GemmSeg seg[kGemmMaxSeg];
   const h1* res_x;  // [M][N] G_RESIDUAL, G_FFN_OUT
   const h1* res_r;  // [M][N] G_FFN_OUT

@@ -31,21 +31,57 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 constexpr int BN = 128;
 constexpr int kGemmThreads = 256;
 // Fused epilogues, shared by the product kernels: acc[i][j] is the 32x32 block (i, j) of the wave's
-// (BM/2) x 64 tile at rows m0 + wm*(BM/2), columns n0 + wn*64; acc[i][j][v] is
+// (32 MI) x (32 NJ) tile whose first element is (row0, col0); acc[i][j][v] is
 // C[row = 8*(v/4) + 4*(lane/32) + v%4][col = lane%32] of the block.
 // FULL: the workgroup's tile lies inside the matrix, nothing is predicated.  (With a predicate per
 // element every store becomes a branch to an out-of-line block; on the 1024 x 6144 product that
 // was 11 of 59 us.)  The epilogue kind is uniform over the launch segment: one switch, and for the
 // kinds that read operands all 16 of a block are requested before the first is used.
-template <int BM, bool FULL>
-__device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg& sg, const f16v (&acc)[BM / 64][2],
-                                                int m0, int n0, int M, int N, int lane, int wm, int wn) {
-  constexpr int MI = BM / 64;
+// sigmoid_h of the 16 accumulators a lane holds of one 32 x 32 block, the same bits at a fraction
+// of the cost.  Called element by element, sigmoid_h makes a wave take its double branch whenever
+// any of its 64 lanes needs it (every other element), and its fp32 estimate alone (expf and a
+// correctly rounded division, ~35 VALU instructions) is 128 x 35 instructions per lane and tile:
+// the sigmoid epilogue of a 128 x 224 tile took 26 us where a plain store takes 2.5 us.
+// Here the estimate is v_exp_f32 and v_rcp_f32.  Its error: t = -x log2(e) is one rounded product,
+// |dt| <= 9e-8 |t|, so exp2(t) is off by at most 6.2e-8 |t| relative, which reaches the result
+// scaled by e/(1+e); over the range that is not handed to the exact path anyway (x > -9.3) that
+// is below 1e-6, plus one ulp each for v_exp_f32, the sum and v_rcp_f32: under 20 fp32 ulps.  An
+// estimate further than 64 ulps from the midpoint of two binary16 values therefore rounds as the
+// exact value does; the others (about 1 in 60) are queued per lane and evaluated in double
+// afterwards, one per lane and pass.
+__device__ __forceinline__ void sigmoid_h16(const f16v& c, h1 (&y)[16]) {
+  h1 x[16];
+  uint32_t pend = 0;
+#pragma unroll
+  for (int v = 0; v < 16; v++) {
+    x[v] = (h1)c[v];
+    const float e = __builtin_amdgcn_exp2f((float)x[v] * -1.44269504088896340736f);
+    const float s32 = __builtin_amdgcn_rcpf(1.0f + e);
+    const uint32_t frac = __float_as_uint(s32) & 0x1FFFu;  // the 13 fp32 mantissa bits binary16 drops
+    const bool safe = s32 > 1e-4f && (frac - (0x1000u - 64u)) > 128u;
+    y[v] = (h1)s32;
+    pend |= safe ? 0u : (1u << v);
+  }
+  while (pend) {
+    const int v = __builtin_ctz(pend);
+    pend &= pend - 1;
+    h1 xv = x[0];
+#pragma unroll
+    for (int u = 1; u < 16; u++) xv = (v == u) ? x[u] : xv;
+    const h1 r = sigmoid_h_exact(xv);
+#pragma unroll
+    for (int u = 0; u < 16; u++) y[u] = (v == u) ? r : y[u];
+  }
+}
+
+template <int MI, int NJ, bool FULL>
+__device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg& sg, const f16v (&acc)[MI][NJ],
+                                                int row0, int col0, int M, int N, int lane) {
   auto for_tile = [&](int i, int j, auto&& f) {
-    const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    const int col = col0 + j * 32 + (lane & 31);
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-      const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+      const int row = row0 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
       if constexpr (FULL)
         f(v, true, (size_t)row * N + col);
       else
@@ -56,7 +92,7 @@ __device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg
 #pragma unroll
     for (int i = 0; i < MI; i++)
 #pragma unroll
-      for (int j = 0; j < 2; j++) g(i, j, acc[i][j]);
+      for (int j = 0; j < NJ; j++) g(i, j, acc[i][j]);
   };
   switch (sg.epi) {
     case G_STORE_F16:
@@ -71,7 +107,9 @@ __device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg
       break;
     case G_SIGMOID:
       for_blocks([&](int i, int j, const f16v& c) {
-        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = sigmoid_h((h1)c[v]); });
+        h1 y[16];
+        sigmoid_h16(c, y);
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = y[v]; });
       });
       break;
     case G_RELU2:
@@ -116,9 +154,9 @@ template <int BM>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, const GemmSeg& sg, const f16v (&acc)[BM / 64][2], int m0,
                                               int n0, int M, int N, int lane, int wm, int wn) {
   if (m0 + BM <= M && n0 + BN <= N)
-    gemm_epilogue_t<BM, true>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+    gemm_epilogue_t<BM / 64, 2, true>(a, sg, acc, m0 + wm * (BM / 2), n0 + wn * 64, M, N, lane);
   else
-    gemm_epilogue_t<BM, false>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+    gemm_epilogue_t<BM / 64, 2, false>(a, sg, acc, m0 + wm * (BM / 2), n0 + wn * 64, M, N, lane);
 }
 
 // BM = 128 (waves 2 x 2 of 64 x 64) or 64 (waves of 32 x 64), for launches that would otherwise
@@ -283,14 +321,19 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
 //
 // LDS layout.  One load instruction brings 8 rows x 64 k = 8 x 128 contiguous bytes (fully
 // coalesced) and lands as 1 KB in lane order: lane l = row l/8, 16-byte slot l%8.  The lane asks
-// for k-segment (l%8) ^ (row%8), so k-segment q of row r sits in slot q ^ (r%8) and the MFMA
-// fragment reads (32 consecutive rows, one k-segment) spread over the banks without padding.
+// for k-segment (l%8) ^ (row%8) ^ (row/8 % 2), so k-segment q of row r sits in slot
+// q ^ (r%8) ^ (r/8 % 2).  A fragment read (32 consecutive rows, one k-segment) is served 16 lanes
+// per cycle over 64 banks; rows r and r+8 lie 1 KB apart, i.e. on the same banks, and the last
+// term moves them one slot apart: SQ_LDS_BANK_CONFLICT is 0 and a read takes 4 cycles (without
+// that term every read was a two-way conflict: 8 cycles).
 // ---------------------------------------------------------------------------
 constexpr int kLdwThreads = 320;
 constexpr int kLdwStages = 4;
 constexpr int kLdwBK = 64;
 static constexpr size_t gemm_ldw_lds_bytes(int bm) { return (size_t)kLdwStages * (bm + BN) * kLdwBK * 2; }
-__device__ __forceinline__ int ldw_at(int row, int q) { return (row >> 3) * 1024 + (row & 7) * 128 + ((q ^ (row & 7)) * 16); }
+__device__ __forceinline__ int ldw_at(int row, int q) {
+  return (row >> 3) * 1024 + (row & 7) * 128 + ((q ^ (row & 7) ^ ((row >> 3) & 1)) * 16);
+}
 
 template <int BM>
 __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
@@ -321,13 +364,13 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
     for (int b = 0; b < kAInstr; b++) {
       int row = m0 + b * 8 + lr;
       row = row < M ? row : M - 1;
-      pa[b] = sg.A + (size_t)row * K + ls * 8;
+      pa[b] = sg.A + (size_t)row * K + (ls ^ (b & 1)) * 8;
     }
 #pragma unroll
     for (int b = 0; b < kBInstr; b++) {
       int row = n0 + b * 8 + lr;
       row = row < N ? row : N - 1;
-      pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + ls * 8;
+      pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + (ls ^ (b & 1)) * 8;
     }
     auto issue = [&](int step) {
       unsigned char* st = gemm_smem + (step % kLdwStages) * kStageBytes;
@@ -405,6 +448,231 @@ static void gemm_ldw_launch(dim3 grid, hipStream_t st, const GemmArgs& a) {
   hipLaunchKernelGGL((gemm_ldw_kernel<BM>), grid, dim3(kLdwThreads), lds, st, a);
 }
 
+// ---------------------------------------------------------------------------
+// binary16 weights, tiles of 128 rows and a width chosen per launch.
+//
+// A launch of 128 x 128 tiles over T = 1024 rows rarely comes out as a whole number of rounds over
+// the compute units (k,v,r of a 2048-wide model: 384 tiles on 256 CUs take as long as 512), and a
+// wider tile moves fewer bytes per product.  Here the host cuts every segment of a launch into
+// tiles of 128 rows x (32 w) columns, w = base or base + 1 per segment, so that the launch has as
+// many workgroups as the part has compute units (or twice, three times as many), and no tile
+// straddles two segments.  The two wave columns of a workgroup take ceil(w/2) and floor(w/2)
+// 32-column blocks; the loops are instantiated per block count, so the products are the same
+// MFMAs in the same k order as in the other kernels and the results are bit-identical.  Loader
+// wave, LDS ring (three or four K-steps of 64, whatever fits 160 KB at the launch's widest tile)
+// and swizzle are those of gemm_ldw_kernel.
+// ---------------------------------------------------------------------------
+constexpr int kVwBM = 128, kVwMaxW = 8, kVwABytes = kVwBM * kLdwBK * 2;
+
+template <int W>
+__device__ __forceinline__ void vw_loader(const GemmSeg& sg, unsigned char* smem, int stage_bytes, int ns, int m0, int n0,
+                                          int M, int N, int K, int lane) {
+  constexpr int kAInstr = kVwABytes / 1024, kBInstr = 4 * W, kPer = kAInstr + kBInstr;
+  static_assert(kPer <= 63, "wait counter");
+  const int lr = lane >> 3, ls = (lane & 7) ^ lr;
+  const h1* pa[kAInstr];
+  const h1* pb[kBInstr];
+#pragma unroll
+  for (int b = 0; b < kAInstr; b++) {
+    int row = m0 + b * 8 + lr;
+    row = row < M ? row : M - 1;
+    pa[b] = sg.A + (size_t)row * K + (ls ^ (b & 1)) * 8;
+  }
+#pragma unroll
+  for (int b = 0; b < kBInstr; b++) {
+    int row = n0 + b * 8 + lr;
+    row = row < N ? row : N - 1;
+    pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + (ls ^ (b & 1)) * 8;
+  }
+  const int nk = K / kLdwBK;
+  auto issue = [&](int step, int slot) {
+    unsigned char* st = smem + slot * stage_bytes;
+    const int k0 = step * kLdwBK;
+#pragma unroll
+    for (int b = 0; b < kAInstr; b++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pa[b] + k0),
+                                       (__attribute__((address_space(3))) void*)(st + b * 1024), 16, 0, 0);
+#pragma unroll
+    for (int b = 0; b < kBInstr; b++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pb[b] + k0),
+                                       (__attribute__((address_space(3))) void*)(st + kVwABytes + b * 1024), 16, 0, 0);
+  };
+  issue(0, 0);
+  if (nk > 1) issue(1, 1);
+  int slot = 2 % ns;
+  for (int k = 0; k < nk; k++) {
+    if (k + 1 < nk)
+      __builtin_amdgcn_s_waitcnt(((kPer >> 4) << 14) | 0x0F70 | (kPer & 15));  // vmcnt(kPer): step k has landed
+    else
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_s_barrier();  // step k may be read; step k-1 has been read by all
+    if (k + 2 < nk) {
+      issue(k + 2, slot);          // ns >= 3: not the slot of step k or k+1
+      slot = slot + 1 == ns ? 0 : slot + 1;
+    }
+  }
+}
+
+template <int NJ>
+__device__ __forceinline__ void vw_mma(const GemmArgs& a, const GemmSeg& sg, const unsigned char* smem, int stage_bytes, int ns,
+                                       int brow0, int m0, int n0, int M, int N, bool full, int lane, int wm) {
+  f16v acc[2][NJ];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+  const int nk = a.K / kLdwBK;
+  int slot = 0;
+  for (int k = 0; k < nk; k++) {
+    __builtin_amdgcn_s_barrier();
+    const unsigned char* st = smem + slot * stage_bytes;
+    slot = slot + 1 == ns ? 0 : slot + 1;
+    h8 fa[4][2], fb[4][NJ];
+#pragma unroll
+    for (int kb = 0; kb < 4; kb++) {
+      const int q = kb * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < 2; i++) fa[kb][i] = *reinterpret_cast<const h8*>(st + ldw_at(wm * 64 + i * 32 + (lane & 31), q));
+#pragma unroll
+      for (int j = 0; j < NJ; j++)
+        fb[kb][j] = *reinterpret_cast<const h8*>(st + kVwABytes + ldw_at(brow0 + j * 32 + (lane & 31), q));
+    }
+#pragma unroll
+    for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kb][i], fb[kb][j], acc[i][j], 0, 0, 0);
+  }
+  if (full)
+    gemm_epilogue_t<2, NJ, true>(a, sg, acc, m0 + wm * 64, n0 + brow0, M, N, lane);
+  else
+    gemm_epilogue_t<2, NJ, false>(a, sg, acc, m0 + wm * 64, n0 + brow0, M, N, lane);
+}
+
+__global__ __launch_bounds__(kLdwThreads) void gemm_vw_kernel(GemmArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
+  // Workgroups are dealt to the eight XCDs in turn (linear index mod 8), each with an L2 of its own.
+  // XCD x therefore takes the x-th eighth of the N tiles, for every strip of rows: it fetches
+  // those weights once and one segment's rows of A, instead of every segment's.  (A matter of
+  // traffic only: any assignment of tiles to workgroups gives the same results.)
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (gridDim.x % 8 == 0) {
+    const int lin = by * gridDim.x + bx, per = gridDim.x / 8;
+    const int r = lin >> 3;
+    bx = (lin & 7) * per + r % per;
+    by = r / per;
+  }
+  int sidx = 0;
+#pragma unroll
+  for (int i = 1; i < kGemmMaxSeg; i++) sidx += (i < a.nseg && bx >= a.tile_start[i]) ? 1 : 0;
+  const GemmSeg& sg = a.seg[sidx];
+  const int ti = bx - a.tile_start[sidx];
+  const int base = a.vw_base[sidx], wide = a.vw_wide[sidx];
+  const int width = base + (ti < wide ? 1 : 0);                  // 32-column blocks of this tile
+  const int n0 = (ti * base + (ti < wide ? ti : wide)) * 32;
+  const int m0 = by * kVwBM;
+  const int M = a.M, K = a.K, N = sg.N;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int stage_bytes = kVwABytes + a.vw_maxw * 4096, ns = a.vw_ns;
+  if (wave == 4) {
+    switch (width) {
+      case 2: vw_loader<2>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 3: vw_loader<3>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 4: vw_loader<4>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 5: vw_loader<5>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 6: vw_loader<6>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 7: vw_loader<7>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      default: vw_loader<8>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+    }
+    return;
+  }
+  const int wm = wave >> 1, wn = wave & 1;
+  const int nj0 = (width + 1) >> 1;
+  const int nj = wn ? width - nj0 : nj0;
+  const int brow0 = wn ? nj0 * 32 : 0;
+  const bool full = m0 + kVwBM <= M && n0 + width * 32 <= N;
+  switch (nj) {
+    case 1: vw_mma<1>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    case 2: vw_mma<2>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    case 3: vw_mma<3>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    default: vw_mma<4>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+  }
+}
+
+// Cuts the launch into tiles for gemm_vw_kernel: the fewest rounds over `cus` compute units whose
+// widest tile is at most kVwMaxW blocks.  false: the launch is too small for tiles of at least
+// 128 x 128 (the other kernels' 64-row tiles serve it better) or too ragged.
+static bool plan_vw(GemmArgs& a, int cus, dim3* grid, size_t* lds) {
+  const int mt = (a.M + kVwBM - 1) / kVwBM;
+  int cb[kGemmMaxSeg], total = 0;
+  for (int s = 0; s < a.nseg; s++) {
+    cb[s] = (a.seg[s].N + 31) / 32;
+    total += cb[s];
+  }
+  for (int rounds = 1; rounds <= 4; rounds++) {
+    const int P = rounds * cus / mt;  // tiles per strip of 128 rows
+    if (P < a.nseg) continue;
+    int t[kGemmMaxSeg], used = 0;
+    for (int s = 0; s < a.nseg; s++) {
+      t[s] = (int)((long)P * cb[s] / total);
+      if (t[s] < 1) t[s] = 1;
+      used += t[s];
+    }
+    if (used > P) continue;
+    // the spare tiles go where the tiles are widest; among equals, to the segment whose epilogue
+    // costs most (a transcendental per element), so that its tiles are the narrow ones
+    auto heavy = [&](int s) { return a.seg[s].epi == G_SIGMOID || a.seg[s].epi == G_SILU ? 1 : 0; };
+    while (used < P) {
+      int best = 0;
+      for (int s = 1; s < a.nseg; s++) {
+        const long l = (long)cb[s] * t[best], r = (long)cb[best] * t[s];
+        if (l > r || (l == r && heavy(s) > heavy(best))) best = s;
+      }
+      t[best]++;
+      used++;
+    }
+    int maxw = 0, minw = INT_MAX;
+    for (int s = 0; s < a.nseg; s++) {
+      const int w = (cb[s] + t[s] - 1) / t[s];
+      maxw = w > maxw ? w : maxw;
+      minw = cb[s] / t[s] < minw ? cb[s] / t[s] : minw;
+    }
+    if (maxw > kVwMaxW) continue;
+    if (minw < 2 || maxw < 4) return false;
+    int tiles = 0;
+    for (int s = 0; s < a.nseg; s++) {
+      a.tile_start[s] = tiles;
+      a.vw_base[s] = cb[s] / t[s];
+      a.vw_wide[s] = cb[s] % t[s];
+      tiles += t[s];
+    }
+    for (int s = a.nseg; s <= kGemmMaxSeg; s++) a.tile_start[s] = INT_MAX;
+    a.tile_start[a.nseg] = tiles;
+    a.vw_maxw = maxw;
+    const size_t stage = kVwABytes + (size_t)maxw * 4096;
+    a.vw_ns = stage * 4 <= 160 * 1024 ? 4 : 3;
+    *lds = stage * a.vw_ns;
+    *grid = dim3(tiles, mt);
+    return true;
+  }
+  return false;
+}
+
+static void gemm_vw_launch(dim3 grid, size_t lds, hipStream_t st, const GemmArgs& a) {
+  static bool raised = false;
+  if (!raised) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_vw_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024);
+    raised = true;
+  }
+  hipLaunchKernelGGL(gemm_vw_kernel, grid, dim3(kLdwThreads), lds, st, a);
+}
+
 static constexpr size_t gemm_lds_bytes(int bm, int bk) { return (size_t)(bm + BN) * (bk + 8) * 2; }
 
 // Tiles above 64 KB of LDS need the limit raised once per kernel.
@@ -467,6 +735,17 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
   // binary16 weights go to the kernel with the loader wave (FRHIP_GEMM_LDW=0 selects the other one:
   // measurement aid); uint8 weights need the registers in between for the dequantisation
   static const bool ldw = !(getenv("FRHIP_GEMM_LDW") && atoi(getenv("FRHIP_GEMM_LDW")) == 0);
+  // FRHIP_GEMM_VW=0 keeps binary16 launches on the fixed 128 / 64 x 128 tiles (measurement aid)
+  static const bool vw = !(getenv("FRHIP_GEMM_VW") && atoi(getenv("FRHIP_GEMM_VW")) == 0);
+  if (!u8 && ldw && vw && !force_bm) {
+    GemmArgs b = a;
+    dim3 grid;
+    size_t lds = 0;
+    if (plan_vw(b, compute_units(), &grid, &lds)) {
+      gemm_vw_launch(grid, lds, st, b);
+      return check_launch(what);
+    }
+  }
   if (!u8 && ldw) {
     if (small)
       gemm_ldw_launch<64>(dim3(tiles, (a.M + 63) / 64), st, a);
@@ -516,4 +795,24 @@ extern "C" int frhip_gemm(const void* x, const frhip_weight* w, void* y, int T, 
   a.K = w->K;
   gemm_add_seg(a, x, w, y, out_dtype == FRHIP_F32 ? G_STORE_F32 : G_STORE_F16);
   return launch_gemm(a, w->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "gemm");
+}
+
+static_assert(FRHIP_ACT_SIGMOID == G_SIGMOID && FRHIP_ACT_RELU2 == G_RELU2 && FRHIP_ACT_SILU == G_SILU, "activation codes");
+
+// matmul + in-place activation (kernels/cuda/ffn_seq.cu:78-81, att_seq.cu:394-395) in one launch.
+extern "C" int frhip_gemm_act(const void* x, const frhip_weight* w, void* y, int T, int act, frhip_stream s) {
+  if (!x || !w || !w->data || !y) return set_error(FRHIP_EINVAL, "gemm_act: null pointer");
+  if (T < 0) return set_error(FRHIP_ESHAPE, "gemm_act: negative T");
+  if (act != FRHIP_ACT_SIGMOID && act != FRHIP_ACT_RELU2 && act != FRHIP_ACT_SILU)
+    return set_error(FRHIP_EINVAL, "gemm_act: act must be SIGMOID, RELU2 or SILU");
+  if (w->dtype != FRHIP_F16 && w->dtype != FRHIP_U8) return set_error(FRHIP_EINVAL, "gemm_act: weight dtype must be F16 or U8");
+  if (w->dtype == FRHIP_U8 && (!w->mx || !w->rx || !w->my || !w->ry)) return set_error(FRHIP_EINVAL, "gemm_act: uint8 weight without mx/rx/my/ry");
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(w->data) % 16 != 0)
+    return set_error(FRHIP_EINVAL, "gemm_act: operands must be 16-byte aligned");
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = T;
+  a.K = w->K;
+  gemm_add_seg(a, x, w, y, act);
+  return launch_gemm(a, w->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "gemm_act");
 }

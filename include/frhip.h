@@ -181,6 +181,15 @@ int frhip_att_one_v5(int C, int H, const void *x, const void *sx, const float *s
 /* matmul, matrix x matrix: kernels/cuda/matmul.cpp:110-121.  x [T][K] binary16, y [T][N] in
  * out_dtype (F16 or F32); fp32 accumulation on the MFMA units.  K must be a multiple of 64. */
 int frhip_gemm(const void *x, const frhip_weight *w, void *y, int T, int out_dtype, frhip_stream s);
+/* matmul followed by the in-place activation the reference applies to its result, as one launch:
+ * y [T][N] binary16 = act(half(x . w)).  act: FRHIP_ACT_SIGMOID (element_wise(InplaceSigmoid),
+ * kernels/cuda/ffn_seq.cu:78-79, att.cu:154-159), FRHIP_ACT_RELU2 (InplaceReLUAndSquare,
+ * ffn_seq.cu:80-81), FRHIP_ACT_SILU (InplaceSiLU, att_seq.cu:394-395, att.cu:145-152).  This is
+ * the epilogue the seq operators below use for r, ffn key and the gate; results are theirs bit for bit. */
+#define FRHIP_ACT_SIGMOID 2
+#define FRHIP_ACT_RELU2 3
+#define FRHIP_ACT_SILU 4
+int frhip_gemm_act(const void *x, const frhip_weight *w, void *y, int T, int act, frhip_stream s);
 
 /* Scratch for the seq-mode operators below: frhip_seq_workspace_bytes(T, C, F) bytes,
  * 256-byte aligned, owned by the caller. */

@@ -26,7 +26,9 @@ def h(x):
     return np.asarray(x, np.float32).astype(np.float16)
 
 
-@pytest.mark.parametrize("T,K,N", [(1024, 2048, 2048), (512, 2560, 8960), (100, 8192, 2048), (1, 64, 128), (130, 128, 200), (7, 1792, 512)])
+@pytest.mark.parametrize("T,K,N", [(1024, 2048, 2048), (512, 2560, 8960), (100, 8192, 2048), (1, 64, 128), (130, 128, 200), (7, 1792, 512),
+                                   # wide enough for the variable-width tiles: ragged N (last block partial), ragged T
+                                   (1024, 256, 7000), (900, 128, 6144)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_gemm_against_oracle(T, K, N, quant):
     x = h(rng.standard_normal((T, K)))
@@ -52,6 +54,38 @@ def test_gemm_against_oracle(T, K, N, quant):
         for t, k in enumerate(ks):
             assert np.array_equal(out[t], wref[k].astype(np.float32)), (t, k)
         assert not out[len(ks):].any()
+
+
+def test_gemm_sigmoid_epilogue_every_binary16_bit_exact():
+    """Every finite binary16 value goes through the product's sigmoid epilogue (identity weight, so the
+    accumulator is the input exactly) and must come out as the oracle's double-evaluated sigmoid, bit for bit;
+    once on 64-row tiles (T = 1024, N = 64) and once on the variable-width tiles (N = 8192, columns repeat)."""
+    bits = np.arange(65536, dtype=np.uint16)
+    x = bits.view(np.float16).copy()
+    x[~np.isfinite(x)] = 0
+    a = x.reshape(1024, 64)
+    want = po.sigmoid_f16(a)
+    for N in (64, 8192):
+        w = np.zeros((64, N), np.float16)
+        w[np.arange(N) % 64, np.arange(N)] = 1
+        pw = fr.PackedWeight(w_kn=w)
+        y = DevBuf.empty((1024, N), np.float16)
+        fr.check(L().frhip_gemm_act(keep(a).ptr, pw.ref, y.ptr, 1024, 2, None))
+        got = y.numpy()
+        for c0 in range(0, N, 64):
+            assert np.array_equal(got[:, c0:c0 + 64].view(np.uint16), want.view(np.uint16)), c0
+
+
+def test_gemm_act_relu2_and_silu_match_the_oracle():
+    x = h(rng.standard_normal((256, 128)))
+    w = h(rng.standard_normal((128, 192)) * 0.1)
+    pw = fr.PackedWeight(w_kn=w)
+    lin = po.gemm_f16(x, w, "f16")
+    y = DevBuf.empty((256, 192), np.float16)
+    fr.check(L().frhip_gemm_act(keep(x).ptr, pw.ref, y.ptr, 256, 3, None))
+    t = lin.astype(np.float16)
+    assert_close_f16(y.numpy(), np.where(t > 0, t * t, np.float16(0)).astype(np.float16), max_ulp=4, max_frac=0.05, what="relu2")  # one spacing of t is two of t*t
+    assert L().frhip_gemm_act(keep(x).ptr, pw.ref, y.ptr, 256, 7, None) == -1
 
 
 def test_gemm_rejects_bad_shapes():
