@@ -5,7 +5,10 @@
 // Both operands are K-contiguous, which is the layout v_mfma_f32_32x32x16_f16 wants:
 // a lane's A (or B) fragment is 8 consecutive k of one row, i.e. one 16-byte load.
 // Workgroup tile 128x128 (64x128 for launches that would otherwise leave CUs idle), 2x2 compute
-// waves of 64x64 (2x2 MFMA tiles, 64 fp32 accumulators per lane).  Two kernels:
+// waves of 64x64 (2x2 MFMA tiles, 64 fp32 accumulators per lane).  Three kernels:
+//   gemm_vw_kernel   binary16 weights, launches large enough for tiles of 128 x 128 and more:
+//                    tile widths are chosen per launch so that the workgroups fill the compute
+//                    units in whole rounds; loader wave and LDS ring as in gemm_ldw_kernel;
 //   gemm_ldw_kernel  binary16 weights: a fifth wave streams the tiles global -> LDS directly
 //                    through a ring of four 64-deep K steps; the compute waves never load;
 //   gemm_kernel      uint8 weights: tiles go global -> registers -> LDS (rows padded by 16 bytes
@@ -449,7 +452,7 @@ static void gemm_ldw_launch(dim3 grid, hipStream_t st, const GemmArgs& a) {
 }
 
 // ---------------------------------------------------------------------------
-// binary16 weights, tiles of 128 rows and a width chosen per launch.
+// binary16 weights, tiles of 128 (or 256) rows and a width chosen per launch.
 //
 // A launch of 128 x 128 tiles over T = 1024 rows rarely comes out as a whole number of rounds over
 // the compute units (k,v,r of a 2048-wide model: 384 tiles on 256 CUs take as long as 512), and a
@@ -460,15 +463,20 @@ static void gemm_ldw_launch(dim3 grid, hipStream_t st, const GemmArgs& a) {
 // 32-column blocks; the loops are instantiated per block count, so the products are the same
 // MFMAs in the same k order as in the other kernels and the results are bit-identical.  Loader
 // wave, LDS ring (three or four K-steps of 64, whatever fits 160 KB at the launch's widest tile)
-// and swizzle are those of gemm_ldw_kernel.
+// and swizzle are those of gemm_ldw_kernel.  gemm_vw_kernel<256> has eight MFMA waves (4 x 2 of
+// 64 rows each) over tiles of 256 rows and at most 160 columns; the host takes it where it saves
+// a round (1024 x 2048 x 10240 as one segment: 58 us against 71 us in two rounds of 128-row tiles).
+// Its predicated epilogue (edge tiles) spills a few registers; the main loop does not.
 // ---------------------------------------------------------------------------
-constexpr int kVwBM = 128, kVwMaxW = 8, kVwABytes = kVwBM * kLdwBK * 2;
+constexpr int kVwMaxW = 8;
 
-template <int W>
+template <int BM, int W>
 __device__ __forceinline__ void vw_loader(const GemmSeg& sg, unsigned char* smem, int stage_bytes, int ns, int m0, int n0,
                                           int M, int N, int K, int lane) {
-  constexpr int kAInstr = kVwABytes / 1024, kBInstr = 4 * W, kPer = kAInstr + kBInstr;
-  static_assert(kPer <= 63, "wait counter");
+  constexpr int kVwABytes = BM * kLdwBK * 2;
+  constexpr int kAInstr = kVwABytes / 1024, kBInstr = 4 * W, kPer = (kAInstr + kBInstr) <= 63 ? (kAInstr + kBInstr) : 0;
+  if constexpr (kPer == 0) return;  // wider than the wait counter allows: the host never plans such a tile
+
   const int lr = lane >> 3, ls = (lane & 7) ^ lr;
   const h1* pa[kAInstr];
   const h1* pb[kBInstr];
@@ -513,9 +521,10 @@ __device__ __forceinline__ void vw_loader(const GemmSeg& sg, unsigned char* smem
   }
 }
 
-template <int NJ>
+template <int BM, int NJ>
 __device__ __forceinline__ void vw_mma(const GemmArgs& a, const GemmSeg& sg, const unsigned char* smem, int stage_bytes, int ns,
                                        int brow0, int m0, int n0, int M, int N, bool full, int lane, int wm) {
+  constexpr int kVwABytes = BM * kLdwBK * 2;
   f16v acc[2][NJ];
 #pragma unroll
   for (int i = 0; i < 2; i++)
@@ -529,23 +538,29 @@ __device__ __forceinline__ void vw_mma(const GemmArgs& a, const GemmSeg& sg, con
     __builtin_amdgcn_s_barrier();
     const unsigned char* st = smem + slot * stage_bytes;
     slot = slot + 1 == ns ? 0 : slot + 1;
-    h8 fa[4][2], fb[4][NJ];
+    // fragments of KG x 16 k are requested together; with eight MFMA waves a lane has 168
+    // registers and holds two of the four k-blocks of a step at a time
+    constexpr int KG = BM == 128 ? 4 : 2;
 #pragma unroll
-    for (int kb = 0; kb < 4; kb++) {
-      const int q = kb * 2 + (lane >> 5);
+    for (int kh = 0; kh < 4; kh += KG) {
+      h8 fa[KG][2], fb[KG][NJ];
 #pragma unroll
-      for (int i = 0; i < 2; i++) fa[kb][i] = *reinterpret_cast<const h8*>(st + ldw_at(wm * 64 + i * 32 + (lane & 31), q));
+      for (int kb = 0; kb < KG; kb++) {
+        const int q = (kh + kb) * 2 + (lane >> 5);
 #pragma unroll
-      for (int j = 0; j < NJ; j++)
-        fb[kb][j] = *reinterpret_cast<const h8*>(st + kVwABytes + ldw_at(brow0 + j * 32 + (lane & 31), q));
-    }
-#pragma unroll
-    for (int kb = 0; kb < 4; kb++)
-#pragma unroll
-      for (int i = 0; i < 2; i++)
+        for (int i = 0; i < 2; i++) fa[kb][i] = *reinterpret_cast<const h8*>(st + ldw_at(wm * 64 + i * 32 + (lane & 31), q));
 #pragma unroll
         for (int j = 0; j < NJ; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kb][i], fb[kb][j], acc[i][j], 0, 0, 0);
+          fb[kb][j] = *reinterpret_cast<const h8*>(st + kVwABytes + ldw_at(brow0 + j * 32 + (lane & 31), q));
+      }
+#pragma unroll
+      for (int kb = 0; kb < KG; kb++)
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < NJ; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kb][i], fb[kb][j], acc[i][j], 0, 0, 0);
+    }
   }
   if (full)
     gemm_epilogue_t<2, NJ, true>(a, sg, acc, m0 + wm * 64, n0 + brow0, M, N, lane);
@@ -553,7 +568,9 @@ __device__ __forceinline__ void vw_mma(const GemmArgs& a, const GemmSeg& sg, con
     gemm_epilogue_t<2, NJ, false>(a, sg, acc, m0 + wm * 64, n0 + brow0, M, N, lane);
 }
 
-__global__ __launch_bounds__(kLdwThreads) void gemm_vw_kernel(GemmArgs a) {
+template <int BM>
+__global__ __launch_bounds__(BM * 2 + 64) void gemm_vw_kernel(GemmArgs a) {
+  constexpr int kVwABytes = BM * kLdwBK * 2, kLoader = BM / 32;  // BM / 32 MFMA waves of 64 rows x half the width, then the loader
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
   // Workgroups are dealt to the eight XCDs in turn (linear index mod 8), each with an L2 of its own.
   // XCD x therefore takes the x-th eighth of the N tiles, for every strip of rows: it fetches
@@ -574,20 +591,20 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_vw_kernel(GemmArgs a) {
   const int base = a.vw_base[sidx], wide = a.vw_wide[sidx];
   const int width = base + (ti < wide ? 1 : 0);                  // 32-column blocks of this tile
   const int n0 = (ti * base + (ti < wide ? ti : wide)) * 32;
-  const int m0 = by * kVwBM;
+  const int m0 = by * BM;
   const int M = a.M, K = a.K, N = sg.N;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int stage_bytes = kVwABytes + a.vw_maxw * 4096, ns = a.vw_ns;
-  if (wave == 4) {
+  if (wave == kLoader) {
     switch (width) {
-      case 2: vw_loader<2>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
-      case 3: vw_loader<3>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
-      case 4: vw_loader<4>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
-      case 5: vw_loader<5>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
-      case 6: vw_loader<6>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
-      case 7: vw_loader<7>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
-      default: vw_loader<8>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 2: vw_loader<BM, 2>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 3: vw_loader<BM, 3>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 4: vw_loader<BM, 4>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 5: vw_loader<BM, 5>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 6: vw_loader<BM, 6>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
+      case 7: vw_loader<BM, BM == 128 ? 7 : 6>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;  // 256 rows: never wider than 5
+      default: vw_loader<BM, BM == 128 ? 8 : 6>(sg, gemm_smem, stage_bytes, ns, m0, n0, M, N, K, lane); break;
     }
     return;
   }
@@ -595,20 +612,22 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_vw_kernel(GemmArgs a) {
   const int nj0 = (width + 1) >> 1;
   const int nj = wn ? width - nj0 : nj0;
   const int brow0 = wn ? nj0 * 32 : 0;
-  const bool full = m0 + kVwBM <= M && n0 + width * 32 <= N;
+  const bool full = m0 + BM <= M && n0 + width * 32 <= N;
   switch (nj) {
-    case 1: vw_mma<1>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
-    case 2: vw_mma<2>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
-    case 3: vw_mma<3>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
-    default: vw_mma<4>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    case 1: vw_mma<BM, 1>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    case 2: vw_mma<BM, 2>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    case 3: vw_mma<BM, 3>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
+    default: vw_mma<BM, BM == 128 ? 4 : 3>(a, sg, gemm_smem, stage_bytes, ns, brow0, m0, n0, M, N, full, lane, wm); break;
   }
 }
 
-// Cuts the launch into tiles for gemm_vw_kernel: the fewest rounds over `cus` compute units whose
-// widest tile is at most kVwMaxW blocks.  false: the launch is too small for tiles of at least
-// 128 x 128 (the other kernels' 64-row tiles serve it better) or too ragged.
-static bool plan_vw(GemmArgs& a, int cus, dim3* grid, size_t* lds) {
-  const int mt = (a.M + kVwBM - 1) / kVwBM;
+// Cuts the launch into tiles of bm rows for gemm_vw_kernel<bm>: the fewest rounds over `cus` compute
+// units whose widest tile fits.  Returns the number of rounds, or 0: the launch is too small for
+// tiles of at least bm x 128 (the other kernels' 64-row tiles serve it better) or too ragged.
+static int plan_vw(GemmArgs& a, int bm, int cus, dim3* grid, size_t* lds) {
+  const int mt = (a.M + bm - 1) / bm;
+  const int abytes = bm * kLdwBK * 2;
+  const int wcap = bm == 128 ? kVwMaxW : 5;  // 256 rows: three stages of (256 + 160) x 64 halves are 156 KB of the 160 KB
   int cb[kGemmMaxSeg], total = 0;
   for (int s = 0; s < a.nseg; s++) {
     cb[s] = (a.seg[s].N + 31) / 32;
@@ -642,8 +661,8 @@ static bool plan_vw(GemmArgs& a, int cus, dim3* grid, size_t* lds) {
       maxw = w > maxw ? w : maxw;
       minw = cb[s] / t[s] < minw ? cb[s] / t[s] : minw;
     }
-    if (maxw > kVwMaxW) continue;
-    if (minw < 2 || maxw < 4) return false;
+    if (maxw > wcap) continue;
+    if (minw < 2 || maxw < 4) return 0;
     int tiles = 0;
     for (int s = 0; s < a.nseg; s++) {
       a.tile_start[s] = tiles;
@@ -654,23 +673,25 @@ static bool plan_vw(GemmArgs& a, int cus, dim3* grid, size_t* lds) {
     for (int s = a.nseg; s <= kGemmMaxSeg; s++) a.tile_start[s] = INT_MAX;
     a.tile_start[a.nseg] = tiles;
     a.vw_maxw = maxw;
-    const size_t stage = kVwABytes + (size_t)maxw * 4096;
+    const size_t stage = abytes + (size_t)maxw * 4096;
     a.vw_ns = stage * 4 <= 160 * 1024 ? 4 : 3;
+    if (stage * a.vw_ns > 160 * 1024) return 0;
     *lds = stage * a.vw_ns;
     *grid = dim3(tiles, mt);
-    return true;
+    return rounds;
   }
-  return false;
+  return 0;
 }
 
+template <int BM>
 static void gemm_vw_launch(dim3 grid, size_t lds, hipStream_t st, const GemmArgs& a) {
   static bool raised = false;
   if (!raised) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_vw_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_vw_kernel<BM>), hipFuncAttributeMaxDynamicSharedMemorySize,
                               160 * 1024);
     raised = true;
   }
-  hipLaunchKernelGGL(gemm_vw_kernel, grid, dim3(kLdwThreads), lds, st, a);
+  hipLaunchKernelGGL((gemm_vw_kernel<BM>), grid, dim3(BM * 2 + 64), lds, st, a);
 }
 
 static constexpr size_t gemm_lds_bytes(int bm, int bk) { return (size_t)(bm + BN) * (bk + 8) * 2; }
@@ -737,12 +758,20 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
   static const bool ldw = !(getenv("FRHIP_GEMM_LDW") && atoi(getenv("FRHIP_GEMM_LDW")) == 0);
   // FRHIP_GEMM_VW=0 keeps binary16 launches on the fixed 128 / 64 x 128 tiles (measurement aid)
   static const bool vw = !(getenv("FRHIP_GEMM_VW") && atoi(getenv("FRHIP_GEMM_VW")) == 0);
+  static const int force_vw_bm = getenv("FRHIP_GEMM_VW_BM") ? atoi(getenv("FRHIP_GEMM_VW_BM")) : 0;  // measurement aid
   if (!u8 && ldw && vw && !force_bm) {
-    GemmArgs b = a;
-    dim3 grid;
-    size_t lds = 0;
-    if (plan_vw(b, compute_units(), &grid, &lds)) {
-      gemm_vw_launch(grid, lds, st, b);
+    // 128-row tiles unless 256-row tiles (eight MFMA waves) need fewer rounds
+    GemmArgs b1 = a, b2 = a;
+    dim3 g1, g2;
+    size_t l1 = 0, l2 = 0;
+    const int r1 = plan_vw(b1, 128, compute_units(), &g1, &l1);
+    const int r2 = force_vw_bm == 128 ? 0 : plan_vw(b2, 256, compute_units(), &g2, &l2);
+    if (r2 && (!r1 || r2 < r1 || force_vw_bm == 256)) {
+      gemm_vw_launch<256>(g2, l2, st, b2);
+      return check_launch(what);
+    }
+    if (r1) {
+      gemm_vw_launch<128>(g1, l1, st, b1);
       return check_launch(what);
     }
   }

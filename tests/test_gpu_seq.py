@@ -28,7 +28,9 @@ def h(x):
 
 @pytest.mark.parametrize("T,K,N", [(1024, 2048, 2048), (512, 2560, 8960), (100, 8192, 2048), (1, 64, 128), (130, 128, 200), (7, 1792, 512),
                                    # wide enough for the variable-width tiles: ragged N (last block partial), ragged T
-                                   (1024, 256, 7000), (900, 128, 6144)])
+                                   (1024, 256, 7000), (900, 128, 6144),
+                                   # one round of 256-row tiles beats two of 128-row tiles: the eight-wave form, full and ragged
+                                   (1024, 128, 10240), (1000, 128, 10000)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_gemm_against_oracle(T, K, N, quant):
     x = h(rng.standard_normal((T, K)))
