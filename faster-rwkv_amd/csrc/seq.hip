@@ -194,20 +194,41 @@ struct Wkv4Seq {
   float *aa_out, *bb_out, *pp_out;
 };
 
+// Steps per batch of loads in the chunk passes: a thread requests the k, v (and r) of kScanB steps
+// before the recurrence touches the first, so a chunk of 16 steps costs one memory round trip
+// instead of 16 (with two waves per SIMD little else hides them: 8.3 -> 6.9 us and 10.7 -> 9.0 us
+// per launch at T = 1024).  What remains is launch, one round trip and the library expf (~28 VALU
+// instructions, six per token and channel over the three passes); a six-instruction exp2-based
+// exponential within 2 ulp brought the three passes from 28.4 to 25.2 us and was not kept: the
+// passes then no longer compute exactly what the one-token kernel does.
+constexpr int kScanB = 16;
+
 __global__ __launch_bounds__(256) void wkv4_local_kernel(Wkv4Seq a) {
   const int c = blockIdx.x * 256 + threadIdx.x, ch = blockIdx.y;
   if (c >= a.C) return;
   const int t0 = ch * a.Lc, t1 = min(t0 + a.Lc, a.T);
   const float w = a.w[c];
   float aa = 0.f, bb = 0.f, pp = -1e30f;
-  for (int t = t0; t < t1; t++) {
-    const float k = a.k[(size_t)t * a.C + c], v = a.v[(size_t)t * a.C + c];
-    const float ww = w + pp;
-    const float p = (ww > k) ? ww : k;
-    const float e1 = expf(ww - p), e2 = expf(k - p);
-    aa = e1 * aa + e2 * v;
-    bb = e1 * bb + e2;
-    pp = p;
+  for (int tb = t0; tb < t1; tb += kScanB) {
+    float kk[kScanB], vv[kScanB];
+#pragma unroll
+    for (int i = 0; i < kScanB; i++) {
+      const int t = tb + i < t1 ? tb + i : t1 - 1;
+      kk[i] = a.k[(size_t)t * a.C + c];
+      vv[i] = a.v[(size_t)t * a.C + c];
+    }
+#pragma unroll
+    for (int i = 0; i < kScanB; i++) {
+      if (tb + i < t1) {
+        const float k = kk[i], v = vv[i];
+        const float ww = w + pp;
+        const float p = (ww > k) ? ww : k;
+        const float e1 = expf(ww - p), e2 = expf(k - p);
+        aa = e1 * aa + e2 * v;
+        bb = e1 * bb + e2;
+        pp = p;
+      }
+    }
   }
   const size_t o = (size_t)ch * a.C + c;
   a.la[o] = aa;
@@ -262,22 +283,36 @@ __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
   const float w = a.w[c], u = a.u[c];
   const size_t o = (size_t)ch * a.C + c;
   float aa = a.sa[o], bb = a.sb[o], pp = a.sp[o];
-  for (int t = t0; t < t1; t++) {
-    const size_t i = (size_t)t * a.C + c;
-    const float k = a.k[i], v = a.v[i];
-    // kernels/cuda/att.cu:43-60
-    float ww = u + k;
-    float p = (pp > ww) ? pp : ww;
-    float e1 = expf(pp - p), e2 = expf(ww - p);
-    const float wkv = (e1 * aa + e2 * v) / (e1 * bb + e2);
-    a.r[i] = a.r[i] * (h1)wkv;
-    ww = w + pp;
-    p = (ww > k) ? ww : k;
-    e1 = expf(ww - p);
-    e2 = expf(k - p);
-    aa = e1 * aa + e2 * v;
-    bb = e1 * bb + e2;
-    pp = p;
+  for (int tb = t0; tb < t1; tb += kScanB) {
+    float kk[kScanB], vv[kScanB];
+    h1 rr[kScanB];
+#pragma unroll
+    for (int i = 0; i < kScanB; i++) {
+      const int t = tb + i < t1 ? tb + i : t1 - 1;
+      const size_t j = (size_t)t * a.C + c;
+      kk[i] = a.k[j];
+      vv[i] = a.v[j];
+      rr[i] = a.r[j];
+    }
+#pragma unroll
+    for (int i = 0; i < kScanB; i++) {
+      if (tb + i < t1) {
+        const float k = kk[i], v = vv[i];
+        // kernels/cuda/att.cu:43-60
+        float ww = u + k;
+        float p = (pp > ww) ? pp : ww;
+        float e1 = expf(pp - p), e2 = expf(ww - p);
+        const float wkv = (e1 * aa + e2 * v) / (e1 * bb + e2);
+        a.r[(size_t)(tb + i) * a.C + c] = rr[i] * (h1)wkv;
+        ww = w + pp;
+        p = (ww > k) ? ww : k;
+        e1 = expf(ww - p);
+        e2 = expf(k - p);
+        aa = e1 * aa + e2 * v;
+        bb = e1 * bb + e2;
+        pp = p;
+      }
+    }
   }
   if (ch == a.nchunk - 1) {
     a.aa_out[c] = aa;
