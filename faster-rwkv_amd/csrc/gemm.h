@@ -45,6 +45,9 @@ constexpr int kDequantRows = 192;
 // uint8 [N][K] -> binary16 [N][K] with the frozen formula (ops.hip)
 int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,
                      hipStream_t st);
+// the same for the nseg matrices of a grouped product (same K), one launch where the shapes allow it
+int dequant_u8_group_async(int nseg, const unsigned char* const* q, const h1* const* mx, const h1* const* rx, const h1* const* my,
+                           const h1* const* ry, h1* const* dst, int K, const int* N, hipStream_t st);
 void gemm_add_seg(GemmArgs& a, const void* A, const frhip_weight* w, void* out, int epi);
 
 }  // namespace frhip

@@ -77,6 +77,42 @@ __device__ __forceinline__ void sigmoid_h16(const f16v& c, h1 (&y)[16]) {
   }
 }
 
+// silu_h of a block's 16 accumulators, the same bits, built like sigmoid_h16.  silu_h rounds
+// e^-x to binary16, adds 1 in binary16 and divides x by the sum in fp32.  The estimates (v_exp_f32
+// for the exponential, v_rcp_f32 for the quotient: under 20 and 3 fp32 ulps off) are taken when
+// they are further than 64 ulps from a binary16 rounding boundary and in the normal binary16
+// range; the other elements are queued and go through silu_h itself.
+__device__ __forceinline__ void silu_h16(const f16v& c, h1 (&y)[16]) {
+  h1 x[16];
+  uint32_t pend = 0;
+  auto far_from_boundary = [](float v) {
+    const uint32_t frac = __float_as_uint(v) & 0x1FFFu;
+    const float m = __builtin_fabsf(v);
+    return m > 1e-4f && m < 60000.f && (frac - (0x1000u - 64u)) > 128u;
+  };
+#pragma unroll
+  for (int v = 0; v < 16; v++) {
+    x[v] = (h1)c[v];
+    const float xf = (float)x[v];
+    const float ef = __builtin_amdgcn_exp2f(xf * -1.44269504088896340736f);
+    const h1 d = (h1)1.0f + (h1)ef;
+    const float qf = xf * __builtin_amdgcn_rcpf((float)d);
+    const bool safe = far_from_boundary(ef) && far_from_boundary(qf);
+    y[v] = (h1)qf;
+    pend |= safe ? 0u : (1u << v);
+  }
+  while (pend) {
+    const int v = __builtin_ctz(pend);
+    pend &= pend - 1;
+    h1 xv = x[0];
+#pragma unroll
+    for (int u = 1; u < 16; u++) xv = (v == u) ? x[u] : xv;
+    const h1 r = silu_h(xv);
+#pragma unroll
+    for (int u = 0; u < 16; u++) y[u] = (v == u) ? r : y[u];
+  }
+}
+
 template <int MI, int NJ, bool FULL>
 __device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg& sg, const f16v (&acc)[MI][NJ],
                                                 int row0, int col0, int M, int N, int lane) {
@@ -125,7 +161,9 @@ __device__ __forceinline__ void gemm_epilogue_t(const GemmArgs& a, const GemmSeg
       break;
     case G_SILU:
       for_blocks([&](int i, int j, const f16v& c) {
-        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = silu_h((h1)c[v]); });
+        h1 y[16];
+        silu_h16(c, y);
+        for_tile(i, j, [&](int v, bool ok, size_t o) { if (ok) static_cast<h1*>(sg.out)[o] = y[v]; });
       });
       break;
     case G_RESIDUAL:
@@ -731,12 +769,18 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
     // costs the launch about 0.4 x 2 T FLOP per weight at the binary16 kernel's rate: from a few hundred rows
     // on, one expansion and the binary16 kernel win.
     h1* dst = static_cast<h1*>(dq);
+    const unsigned char* qs[kGemmMaxSeg];
+    const h1 *mxs[kGemmMaxSeg], *rxs[kGemmMaxSeg], *mys[kGemmMaxSeg], *rys[kGemmMaxSeg];
+    h1* dsts[kGemmMaxSeg];
+    int ns[kGemmMaxSeg];
     for (int s = 0; s < a.nseg; s++) {
       GemmSeg& g = a.seg[s];
-      if (int rc = dequant_u8_async(g.B, g.mx, g.rx, g.my, g.ry, dst, a.K, g.N, st)) return rc;
+      qs[s] = g.B; mxs[s] = g.mx; rxs[s] = g.rx; mys[s] = g.my; rys[s] = g.ry; ns[s] = g.N;
+      dsts[s] = dst;
       g.B = reinterpret_cast<const unsigned char*>(dst);
       dst += (size_t)g.N * a.K;
     }
+    if (int rc = dequant_u8_group_async(a.nseg, qs, mxs, rxs, mys, rys, dsts, a.K, ns, st)) return rc;
     u8 = false;
   }
   int tiles = 0;

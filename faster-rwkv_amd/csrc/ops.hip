@@ -143,6 +143,56 @@ __global__ void dequant_u8_kernel(const uint32_t* __restrict__ q, const h1* __re
   out[i] = (h4){lo.x, lo.y, hi.x, hi.y};
 }
 
+// The same, 16 codes per thread (K a multiple of 16): one 16-byte load of codes, two each of ry
+// and my, two 16-byte stores.  The seq-mode products expand a launch's uint8 weights with this
+// before the binary16 GEMM, so it runs at copy rate or the expansion eats what it saves: with
+// 4 codes per thread (a 64-bit division, eight 2-byte loads of ry/my per word) the 2560 x 2560
+// matrices of a 3B model took 8.0 us each, 2.4 TB/s of traffic.
+__device__ __forceinline__ void dequant_chunk16(const u32x4* __restrict__ q, const h1* __restrict__ mx, const h1* __restrict__ rx,
+                                                const h1* __restrict__ my, const h1* __restrict__ ry, h8* __restrict__ out,
+                                                int K16, unsigned i) {
+  const unsigned n = i / (unsigned)K16;
+  const int k = (int)(i - n * (unsigned)K16) * 16;
+  const float c2 = dequant_c(rx[n]);
+  const float m2 = (float)mx[n];
+  const u32x4 w = __builtin_nontemporal_load(q + i);
+#pragma unroll
+  for (int hh = 0; hh < 2; hh++) {
+    const h8 ryv = *reinterpret_cast<const h8*>(ry + k + hh * 8);
+    const h8 myv = *reinterpret_cast<const h8*>(my + k + hh * 8);
+    const uint32_t w0 = w[2 * hh], w1 = w[2 * hh + 1];
+    const h2 p0 = dequant_pair<0>(w0, c2, m2, ryv.s01, myv.s01);
+    const h2 p1 = dequant_pair<1>(w0, c2, m2, ryv.s23, myv.s23);
+    const h2 p2 = dequant_pair<0>(w1, c2, m2, ryv.s45, myv.s45);
+    const h2 p3 = dequant_pair<1>(w1, c2, m2, ryv.s67, myv.s67);
+    out[(size_t)i * 2 + hh] = (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+  }
+}
+
+__global__ __launch_bounds__(256) void dequant_u8x16_kernel(const u32x4* __restrict__ q, const h1* __restrict__ mx,
+                                                            const h1* __restrict__ rx, const h1* __restrict__ my,
+                                                            const h1* __restrict__ ry, h8* __restrict__ out, int K16,
+                                                            unsigned chunks) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;  // index of a 16-code chunk
+  if (i < chunks) dequant_chunk16(q, mx, rx, my, ry, out, K16, i);
+}
+
+// Up to four matrices over the same K in one launch (blockIdx.y picks the matrix): the weights of
+// a grouped product (k, v, r, g or ffn r, k) are expanded together instead of in four launches of
+// a few microseconds each.
+struct DequantGroup {
+  const u32x4* q[4];
+  const h1 *mx[4], *rx[4], *my[4], *ry[4];
+  h8* out[4];
+  unsigned chunks[4];
+  int K16;
+};
+__global__ __launch_bounds__(256) void dequant_u8x16_group_kernel(DequantGroup g) {
+  const int s = blockIdx.y;
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i < g.chunks[s]) dequant_chunk16(g.q[s], g.mx[s], g.rx[s], g.my[s], g.ry[s], g.out[s], g.K16, i);
+}
+
 __global__ __launch_bounds__(256) void copy_probe_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t n) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
@@ -250,10 +300,46 @@ __global__ __launch_bounds__(1024) void argmax_f32_kernel(const float* __restric
 
 int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,
                      hipStream_t st) {
+  const size_t chunks = (size_t)N * (K / 16);
+  if (K % 16 == 0 && chunks < (1u << 31) && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(ry) % 16 == 0 && reinterpret_cast<uintptr_t>(my) % 16 == 0) {
+    hipLaunchKernelGGL(dequant_u8x16_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, (const u32x4*)q, mx, rx, my, ry,
+                       (h8*)dst, K / 16, (unsigned)chunks);
+    return check_launch("dequant_u8");
+  }
   const size_t words = (size_t)N * (K / 4);
   hipLaunchKernelGGL(dequant_u8_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, (const uint32_t*)q, mx, rx, my, ry,
                      (h4*)dst, K, N);
   return check_launch("dequant_u8");
+}
+
+int dequant_u8_group_async(int nseg, const unsigned char* const* q, const h1* const* mx, const h1* const* rx, const h1* const* my,
+                           const h1* const* ry, h1* const* dst, int K, const int* N, hipStream_t st) {
+  bool fast = K % 16 == 0 && nseg >= 2 && nseg <= 4;
+  unsigned most = 0;
+  DequantGroup g;
+  for (int s = 0; fast && s < nseg; s++) {
+    const size_t chunks = (size_t)N[s] * (K / 16);
+    fast = chunks < (1u << 31) && reinterpret_cast<uintptr_t>(q[s]) % 16 == 0 && reinterpret_cast<uintptr_t>(dst[s]) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(ry[s]) % 16 == 0 && reinterpret_cast<uintptr_t>(my[s]) % 16 == 0;
+    g.q[s] = reinterpret_cast<const u32x4*>(q[s]);
+    g.mx[s] = mx[s]; g.rx[s] = rx[s]; g.my[s] = my[s]; g.ry[s] = ry[s];
+    g.out[s] = reinterpret_cast<h8*>(dst[s]);
+    g.chunks[s] = (unsigned)chunks;
+    most = g.chunks[s] > most ? g.chunks[s] : most;
+  }
+  if (!fast) {
+    for (int s = 0; s < nseg; s++)
+      if (int rc = dequant_u8_async(q[s], mx[s], rx[s], my[s], ry[s], dst[s], K, N[s], st)) return rc;
+    return 0;
+  }
+  for (int s = nseg; s < 4; s++) {
+    g.q[s] = g.q[0]; g.mx[s] = g.mx[0]; g.rx[s] = g.rx[0]; g.my[s] = g.my[0]; g.ry[s] = g.ry[0]; g.out[s] = g.out[0];
+    g.chunks[s] = 0;
+  }
+  g.K16 = K / 16;
+  hipLaunchKernelGGL(dequant_u8x16_group_kernel, dim3((most + 255) / 256, nseg), dim3(256), 0, st, g);
+  return check_launch("dequant_u8 (group)");
 }
 
 }  // namespace frhip

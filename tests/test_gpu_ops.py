@@ -111,9 +111,9 @@ def test_dequant_all_codes_bit_exact():
             assert (np.abs(y.numpy() - exact) <= 4e-7 * (terms[0] + terms[1] + terms[2]) + 1e-30).all(), k
 
 
-def test_dequant_random_matrix_bit_exact():
+@pytest.mark.parametrize("K,N", [(2048, 320), (2560, 100), (36, 7)])  # 16 codes per thread; K % 16 != 0: 4 per thread
+def test_dequant_random_matrix_bit_exact(K, N):
     from synth import quantize_u8
-    K, N = 2048, 320
     w = h(rng.standard_normal((K, N)) * 0.02)
     q, mx, rx, my, ry = quantize_u8(w)
     pw = PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry)

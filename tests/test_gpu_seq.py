@@ -58,24 +58,27 @@ def test_gemm_against_oracle(T, K, N, quant):
         assert not out[len(ks):].any()
 
 
-def test_gemm_sigmoid_epilogue_every_binary16_bit_exact():
+def test_gemm_sigmoid_and_silu_epilogues_every_binary16_bit_exact():
     """Every finite binary16 value goes through the product's sigmoid epilogue (identity weight, so the
-    accumulator is the input exactly) and must come out as the oracle's double-evaluated sigmoid, bit for bit;
+    accumulator is the input exactly) and must come out as the oracle's double-evaluated sigmoid (and its silu), bit for bit;
     once on 64-row tiles (T = 1024, N = 64) and once on the variable-width tiles (N = 8192, columns repeat)."""
     bits = np.arange(65536, dtype=np.uint16)
     x = bits.view(np.float16).copy()
     x[~np.isfinite(x)] = 0
+    x[bits == 0x8000] = 0  # the accumulator of 0 + (-0)(1) is +0: -0 cannot reach the epilogue this way
     a = x.reshape(1024, 64)
     want = po.sigmoid_f16(a)
+    want_silu = po.silu_f16(a)
     for N in (64, 8192):
         w = np.zeros((64, N), np.float16)
         w[np.arange(N) % 64, np.arange(N)] = 1
         pw = fr.PackedWeight(w_kn=w)
         y = DevBuf.empty((1024, N), np.float16)
-        fr.check(L().frhip_gemm_act(keep(a).ptr, pw.ref, y.ptr, 1024, 2, None))
-        got = y.numpy()
-        for c0 in range(0, N, 64):
-            assert np.array_equal(got[:, c0:c0 + 64].view(np.uint16), want.view(np.uint16)), c0
+        for act, ref in ((2, want), (4, want_silu)):  # FRHIP_ACT_SIGMOID, FRHIP_ACT_SILU
+            fr.check(L().frhip_gemm_act(keep(a).ptr, pw.ref, y.ptr, 1024, act, None))
+            got = y.numpy()
+            for c0 in range(0, N, 64):
+                assert np.array_equal(got[:, c0:c0 + 64].view(np.uint16), ref.view(np.uint16)), (act, c0)
 
 
 def test_gemm_act_relu2_and_silu_match_the_oracle():
