@@ -76,8 +76,11 @@ __global__ __launch_bounds__(256) void ln_mix_seq_kernel(LnMixSeq a) {
 // The same for C % 8 == 0, C <= 8 * 256 * NG: a workgroup takes kLnRows consecutive rows plus the
 // row before them (the token shift of its first row), every thread owns NG groups of 8 elements
 // of every row in registers, all rows are loaded up front and their statistics reduced together
-// (two barriers per workgroup), and the mixed rows leave as 16-byte stores.
-constexpr int kLnRows = 4;
+// (two barriers per workgroup), and the mixed rows leave as 16-byte stores.  The launch is a chain
+// of one load, two reductions and one store per workgroup, so what counts is how many workgroups
+// a compute unit has to overlap: at T = 1024, C = 2048 four rows per workgroup (one workgroup per
+// CU, every row read 1.25 times) take 8.7 us, two 7.4 us, one (every row read twice) 7.0 us.
+constexpr int kLnRows = 1;
 
 template <int NG>
 __global__ __launch_bounds__(256) void ln_mix_rows_kernel(LnMixSeq a) {
