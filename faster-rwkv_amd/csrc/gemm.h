@@ -32,6 +32,11 @@ struct GemmArgs {
   // gemm_vw_kernel: a segment's tiles are vw_base (the first vw_wide of them vw_base + 1) blocks of 32 columns wide
   int vw_base[kGemmMaxSeg], vw_wide[kGemmMaxSeg], vw_maxw, vw_ns;
   GemmSeg seg[kGemmMaxSeg];
+  // split K (single-segment launches of gemm_ldw_kernel<128> only): slice z of ksplit accumulates K / ksplit of the
+  // product into partial + z * partial_stride as fp32 [M][N]; gemm_splitk_reduce_kernel adds the slices and applies the epilogue
+  int ksplit;
+  float* partial;
+  size_t partial_stride;
   const h1* res_x;  // [M][N] G_RESIDUAL, G_FFN_OUT
   const h1* res_r;  // [M][N] G_FFN_OUT
   int div2;
@@ -40,7 +45,9 @@ struct GemmArgs {
 // dq: optional scratch of gemm_dequant_bytes(a) bytes.  With it, uint8 weights of a launch with at least
 // kDequantRows rows are expanded once to binary16 (the standalone dequantisation: the same bits as the
 // in-kernel one) and the launch takes the binary16 kernel.
-int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq = nullptr);
+// partial: optional fp32 scratch of max_split slices of partial_stride floats (>= M * N each) for splitting K.
+int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq = nullptr, float* partial = nullptr,
+                size_t partial_stride = 0, int max_split = 0);
 constexpr int kDequantRows = 192;
 // uint8 [N][K] -> binary16 [N][K] with the frozen formula (ops.hip)
 int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,

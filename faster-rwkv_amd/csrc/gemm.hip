@@ -17,7 +17,8 @@
 //                    formula as the standalone dequantisation, so the product sees exactly the
 //                    dequantised matrix.
 // Products are exact in fp32, accumulation is fp32 in ascending k, and the result is rounded once
-// to the output type (kernels/cuda/matmul.cpp:38-42,64-68); both kernels give the same bits.
+// to the output type (kernels/cuda/matmul.cpp:38-42,64-68); all kernels give the same bits, except
+// that a launch split over K (launch_gemm) adds its slices' fp32 sums at the end.
 // Independent products over the same T and K share one launch ("segments"), each with
 // its own X, W and fused epilogue.
 #include <climits>
@@ -30,6 +31,7 @@
 namespace frhip {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f4v __attribute__((ext_vector_type(4)));
 
 constexpr int BN = 128;
 constexpr int kGemmThreads = 256;
@@ -393,7 +395,9 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
   const int M = a.M, K = a.K, N = sg.N;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nk = K / kLdwBK;
+  const int ksplit = a.ksplit > 1 ? a.ksplit : 1;
+  const int nk = K / kLdwBK / ksplit;                   // K-steps of this slice
+  const int kbase = (int)blockIdx.z * nk * kLdwBK;
 
   if (wave == 4) {
     // ---- the loader ----
@@ -405,13 +409,13 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
     for (int b = 0; b < kAInstr; b++) {
       int row = m0 + b * 8 + lr;
       row = row < M ? row : M - 1;
-      pa[b] = sg.A + (size_t)row * K + (ls ^ (b & 1)) * 8;
+      pa[b] = sg.A + (size_t)row * K + kbase + (ls ^ (b & 1)) * 8;
     }
 #pragma unroll
     for (int b = 0; b < kBInstr; b++) {
       int row = n0 + b * 8 + lr;
       row = row < N ? row : N - 1;
-      pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + (ls ^ (b & 1)) * 8;
+      pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + kbase + (ls ^ (b & 1)) * 8;
     }
     auto issue = [&](int step) {
       unsigned char* st = gemm_smem + (step % kLdwStages) * kStageBytes;
@@ -474,7 +478,59 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
         for (int j = 0; j < 2; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kb][i], fb[kb][j], acc[i][j], 0, 0, 0);
   }
-  gemm_epilogue<BM>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+  if (a.ksplit > 1) {
+    GemmSeg sp = sg;  // this slice's sums go out as fp32; the epilogue proper follows in gemm_splitk_reduce_kernel
+    sp.out = a.partial + (size_t)blockIdx.z * a.partial_stride;
+    sp.epi = G_STORE_F32;
+    gemm_epilogue<BM>(a, sp, acc, m0, n0, M, N, lane, wm, wn);
+  } else {
+    gemm_epilogue<BM>(a, sg, acc, m0, n0, M, N, lane, wm, wn);
+  }
+}
+
+// Adds the K slices of a split launch in slice order and applies the launch's epilogue; a thread
+// takes 8 consecutive outputs of a row (N % 8 == 0).
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a) {
+  const GemmSeg& sg = a.seg[0];
+  const size_t total = (size_t)a.M * sg.N;
+  const size_t o = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (o >= total) return;
+  float acc[8];
+  {
+    const f4v p0 = *reinterpret_cast<const f4v*>(a.partial + o), p1 = *reinterpret_cast<const f4v*>(a.partial + o + 4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) { acc[i] = p0[i]; acc[4 + i] = p1[i]; }
+  }
+  for (int z = 1; z < a.ksplit; z++) {
+    const float* p = a.partial + (size_t)z * a.partial_stride + o;
+    const f4v p0 = *reinterpret_cast<const f4v*>(p), p1 = *reinterpret_cast<const f4v*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) { acc[i] += p0[i]; acc[4 + i] += p1[i]; }
+  }
+  if (sg.epi == G_STORE_F32) {
+    float* out = static_cast<float*>(sg.out) + o;
+#pragma unroll
+    for (int i = 0; i < 8; i++) out[i] = acc[i];
+    return;
+  }
+  h8 y;
+  if (sg.epi == G_STORE_F16) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = (h1)acc[i];
+  } else if (sg.epi == G_RESIDUAL) {
+    const h8 x = *reinterpret_cast<const h8*>(a.res_x + o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = x[i] + (h1)acc[i];
+  } else {  // G_FFN_OUT
+    const h8 x = *reinterpret_cast<const h8*>(a.res_x + o), r = *reinterpret_cast<const h8*>(a.res_r + o);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      h1 v = __builtin_fmaf16((h1)acc[i], r[i], x[i]);
+      if (a.div2) v = v / (h1)2.0f;
+      y[i] = v;
+    }
+  }
+  *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o) = y;
 }
 
 template <int BM>
@@ -761,7 +817,8 @@ static int env_bk() {
   return e ? atoi(e) : 0;
 }
 
-int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq) {
+int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq, float* partial, size_t partial_stride,
+                int max_split) {
   if (a.M <= 0) return 0;
   if (a.K <= 0 || a.K % 64 != 0) return set_error(FRHIP_ESHAPE, "gemm: K must be a positive multiple of 64");
   if (u8 && dq && a.M >= kDequantRows) {
@@ -800,6 +857,30 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
   // binary16 weights go to the kernel with the loader wave (FRHIP_GEMM_LDW=0 selects the other one:
   // measurement aid); uint8 weights need the registers in between for the dequantisation
   static const bool ldw = !(getenv("FRHIP_GEMM_LDW") && atoi(getenv("FRHIP_GEMM_LDW")) == 0);
+  // Split K: a single product with few outputs and a long K (ffn value: 1024 x 8192 x 2048) fills the compute units only
+  // with 64 x 128 tiles, which ask L2 for 1.5 times the bytes of 128 x 128 tiles per product and are bound by just that
+  // (786 MB in 57 us).  With scratch for the partial sums the launch runs ksplit slices of K over 128 x 128 tiles, and a
+  // second kernel adds the slices in order and applies the epilogue.  The sums are grouped by slice, so the result can
+  // differ from the unsplit launch in the last fp32 bit before the rounding to binary16.  FRHIP_GEMM_SPLITK=0: off.
+  static const bool splitk = !(getenv("FRHIP_GEMM_SPLITK") && atoi(getenv("FRHIP_GEMM_SPLITK")) == 0);
+  if (!u8 && ldw && splitk && !force_bm && partial && max_split >= 2 && a.nseg == 1 && a.K >= 4096 && a.seg[0].N % 8 == 0 &&
+      (a.seg[0].epi == G_STORE_F16 || a.seg[0].epi == G_STORE_F32 || a.seg[0].epi == G_RESIDUAL || a.seg[0].epi == G_FFN_OUT) &&
+      (size_t)a.M * a.seg[0].N <= partial_stride) {
+    const long t128 = (long)tiles * m128;
+    int S = (int)(compute_units() / t128);
+    if (S > max_split) S = max_split;
+    while (S >= 2 && (a.K % (kLdwBK * S) != 0 || a.K / (kLdwBK * S) < 16)) S--;
+    if (S >= 2 && t128 * S * 4 >= (long)compute_units() * 3) {  // the slices fill at least three quarters of the CUs
+      a.ksplit = S;
+      a.partial = partial;
+      a.partial_stride = partial_stride;
+      gemm_ldw_launch<128>(dim3(tiles, m128, S), st, a);
+      if (int rc = check_launch(what)) return rc;
+      const size_t threads = ((size_t)a.M * a.seg[0].N + 7) / 8;
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
+      return check_launch(what);
+    }
+  }
   // FRHIP_GEMM_VW=0 keeps binary16 launches on the fixed 128 / 64 x 128 tiles (measurement aid)
   static const bool vw = !(getenv("FRHIP_GEMM_VW") && atoi(getenv("FRHIP_GEMM_VW")) == 0);
   static const int force_vw_bm = getenv("FRHIP_GEMM_VW_BM") ? atoi(getenv("FRHIP_GEMM_VW_BM")) : 0;  // measurement aid

@@ -601,7 +601,8 @@ extern "C" int frhip_ffn_seq(int T, int C, int F, const void* x, const void* sx,
   b.M = T; b.K = F;
   b.res_x = (const h1*)x; b.res_r = w.m2; b.div2 = post_div2 ? 1 : 0;
   gemm_add_seg(b, w.vx, vw, x_out, G_FFN_OUT);
-  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v", w.dq);
+  // the four fp32 [T][C] buffers of the workspace (unused by ffn) take the partial sums of a K-split launch
+  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v", w.dq, w.f0, (size_t)(w.f1 - w.f0), 4);
 }
 
 // RWKV-4 sequence attention.  The reference has no such operator
