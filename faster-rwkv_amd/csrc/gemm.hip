@@ -891,6 +891,31 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
     size_t l1 = 0, l2 = 0;
     const int r1 = plan_vw(b1, 128, compute_units(), &g1, &l1);
     const int r2 = force_vw_bm == 128 ? 0 : plan_vw(b2, 256, compute_units(), &g2, &l2);
+    // A grouped launch that needs two rounds although each of its products alone fits one (ffn r,k at T = 1024:
+    // 2048 columns in one round of 64 x 128 tiles, 8192 in one round of 128 x 256) goes out as separate launches.
+    static const bool separate = !(getenv("FRHIP_GEMM_SEPARATE") && atoi(getenv("FRHIP_GEMM_SEPARATE")) == 0);
+    if (separate && a.nseg > 1 && (r1 == 0 || r1 >= 2) && (r2 == 0 || r2 >= 2)) {
+      bool each_one_round = true;
+      for (int sgi = 0; sgi < a.nseg && each_one_round; sgi++) {
+        GemmArgs one = a;
+        one.nseg = 1;
+        one.seg[0] = a.seg[sgi];
+        dim3 g;
+        size_t l = 0;
+        const int rr1 = plan_vw(one, 128, compute_units(), &g, &l), rr2 = plan_vw(one, 256, compute_units(), &g, &l);
+        const long t64 = (long)((a.seg[sgi].N + BN - 1) / BN) * ((a.M + 63) / 64);
+        each_one_round = rr1 == 1 || rr2 == 1 || (rr1 == 0 && rr2 == 0 && t64 <= compute_units());
+      }
+      if (each_one_round) {
+        for (int sgi = 0; sgi < a.nseg; sgi++) {
+          GemmArgs one = a;
+          one.nseg = 1;
+          one.seg[0] = a.seg[sgi];
+          if (int rc = launch_gemm(one, false, st, what, nullptr, nullptr, 0, 0)) return rc;
+        }
+        return 0;
+      }
+    }
     if (r2 && (!r1 || r2 < r1 || force_vw_bm == 256)) {
       gemm_vw_launch<256>(g2, l2, st, b2);
       return check_launch(what);
