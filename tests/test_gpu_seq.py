@@ -104,7 +104,9 @@ def _common(C_):
     return (h(1 + 0.1 * rng.standard_normal(C_)), h(0.1 * rng.standard_normal(C_)))
 
 
-@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1, 512, 1024), (33, 768, 3072)])
+# (1024, 2048, 8192): r and k as separate one-round launches, the value product split over K in two slices;
+# (300, 2048, 8192): the value product in four slices over ragged row tiles
+@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1024, 2048, 8192), (1, 512, 1024), (33, 768, 3072)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_ffn_seq(T, C_, F_, quant):
     if quant and C_ == 2048:
