@@ -395,9 +395,11 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
   const int M = a.M, K = a.K, N = sg.N;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // slice z of ksplit takes K-steps [z base + min(z, rem), ...): the first rem slices one step more
   const int ksplit = a.ksplit > 1 ? a.ksplit : 1;
-  const int nk = K / kLdwBK / ksplit;                   // K-steps of this slice
-  const int kbase = (int)blockIdx.z * nk * kLdwBK;
+  const int kz = blockIdx.z, ksteps = K / kLdwBK, kper = ksteps / ksplit, krem = ksteps % ksplit;
+  const int nk = kper + (kz < krem ? 1 : 0);            // K-steps of this slice
+  const int kbase = (kz * kper + (kz < krem ? kz : krem)) * kLdwBK;
 
   if (wave == 4) {
     // ---- the loader ----
@@ -869,8 +871,8 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
     const long t128 = (long)tiles * m128;
     int S = (int)(compute_units() / t128);
     if (S > max_split) S = max_split;
-    while (S >= 2 && (a.K % (kLdwBK * S) != 0 || a.K / (kLdwBK * S) < 16)) S--;
-    if (S >= 2 && t128 * S * 4 >= (long)compute_units() * 3) {  // the slices fill at least three quarters of the CUs
+    while (S >= 2 && a.K / (kLdwBK * S) < 16) S--;
+    if (S >= 2 && t128 * S * 5 >= (long)compute_units() * 3) {  // the slices fill at least 60 % of the CUs
       a.ksplit = S;
       a.partial = partial;
       a.partial_stride = partial_stride;

@@ -105,18 +105,19 @@ def _common(C_):
 
 
 # (1024, 2048, 8192): r and k as separate one-round launches, the value product split over K in two slices;
-# (300, 2048, 8192): the value product in four slices over ragged row tiles
-@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1024, 2048, 8192), (1, 512, 1024), (33, 768, 3072)])
+# (300, 2048, 8192): the value product in four slices over ragged row tiles; (512, 2560, 8960): three slices of 47, 47 and 46 K-steps
+@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1024, 2048, 8192), (512, 2560, 8960), (1, 512, 1024), (33, 768, 3072)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_ffn_seq(T, C_, F_, quant):
-    if quant and C_ == 2048:
+    if quant and C_ >= 2048:
         pytest.skip("covered by the fp16 case at this size; uint8 covered at the smaller sizes")
-    x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
-    ln_w, ln_b = _common(C_)
-    mk, mr = h(rng.uniform(0, 1, C_)), h(rng.uniform(0, 1, C_))
-    kw, kref = make_weight(h(rng.standard_normal((C_, F_)) * 0.02), quant)
-    vw, vref = make_weight(h(rng.standard_normal((F_, C_)) * 0.02), quant)
-    rw, rref = make_weight(h(rng.standard_normal((C_, C_)) * 0.02), quant)
+    g = np.random.default_rng(5000 + T) if T >= 512 else rng  # the full-size cases draw from a stream of their own
+    x, sx = h(g.standard_normal((T, C_)) * 2), h(g.standard_normal(C_))
+    ln_w, ln_b = h(1 + 0.1 * g.standard_normal(C_)), h(0.1 * g.standard_normal(C_))
+    mk, mr = h(g.uniform(0, 1, C_)), h(g.uniform(0, 1, C_))
+    kw, kref = make_weight(h(g.standard_normal((C_, F_)) * 0.02), quant)
+    vw, vref = make_weight(h(g.standard_normal((F_, C_)) * 0.02), quant)
+    rw, rref = make_weight(h(g.standard_normal((C_, C_)) * 0.02), quant)
     ref_x, ref_xx = po.ffn_f16(x, sx, ln_w, ln_b, mk, mr, kref, vref, rref)
     x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
     ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, F_))
