@@ -85,6 +85,7 @@ _SIGS = {
     "frhip_decode_workspace_bytes": (_sz, [_i, _i]),
     "frhip_att_one_v4": (_i, [_i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),
     "frhip_ffn_one": (_i, [_i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
+    "frhip_ffn_one_static": (_i, [_i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp]),
     "frhip_head": (_i, [_i, _vp, _vp, _vp, _WP, _vp, _vp]),
     "frhip_head_mirror": (_i, [_i, _vp, _vp, _vp, _WP, _vp, _vp, _vp]),
     "frhip_att_one_v5_1": (_i, [_i, _i] + [_vp] * 13 + [_WP] * 5 + [_vp] * 5),

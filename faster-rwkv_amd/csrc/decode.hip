@@ -25,6 +25,7 @@
 #include <climits>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "device_utils.h"
@@ -1140,6 +1141,40 @@ Workspace carve(void* ws, int C) {
 }
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// Scratch for frhip_ffn_one_static: the workspace of frhip_ffn_one for the largest shape
+// that entry point accepts, as a file-scope device array.  Every GPU the library runs on holds
+// its own copy (112 KB) until the process ends.  Host code never uses the array's name as an
+// address: the device address is looked up once per device with hipGetSymbolAddress and kept.
+// ---------------------------------------------------------------------------
+namespace frhip {
+constexpr int kStaticMaxC = 4096;
+constexpr int kStaticMaxF = 16384;
+// frhip_decode_workspace_bytes(kStaticMaxC, kStaticMaxF): 4 x 8 KB + 32 KB + 3 x 16 KB
+constexpr size_t kStaticScratchBytes = 4 * 8192 + 32768 + 3 * 16384;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, once looked up
+static std::mutex g_scratch_mu;
+
+// Looks up the current device's copy of `scratch` (once per device) and returns it in *ptr.
+int static_scratch(void** ptr) {
+  int dev = -1;
+  FR_TRY(hip_result(hipGetDevice(&dev), "hipGetDevice"));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(FRHIP_EINVAL, "device index beyond the static scratch table");
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    FR_TRY(hip_result(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)"));
+    if (!p || reinterpret_cast<uintptr_t>(p) % 256 != 0) return set_error(FRHIP_ESTATE, "static scratch has no usable device address");
+    g_scratch_ptr[dev] = p;
+  }
+  if (ptr) *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace frhip
+
 extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const float* aa, const float* bb,
                                 const float* pp, const void* ln_w, const void* ln_b, const void* k_mix,
                                 const void* v_mix, const void* r_mix, const float* t_decay, const float* t_first,
@@ -1341,6 +1376,20 @@ extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const 
   b.div2 = post_div2 ? 1 : 0;
   add_seg(b, vw, 0, E_FFN_OUT, x_out);
   return launch_rows(b, vw->dtype == FRHIP_U8, st, "ffn_out");
+}
+
+extern "C" int frhip_ffn_one_static(int C, int F, const void* x, const void* sx, const void* ln_w, const void* ln_b,
+                                    const void* k_mix, const void* r_mix, const frhip_weight* kw,
+                                    const frhip_weight* vw, const frhip_weight* rw, void* x_out, void* xx_out,
+                                    int post_div2, frhip_stream s) {
+  if (C > kStaticMaxC || F > kStaticMaxF)
+    return set_error(FRHIP_ESHAPE, "ffn_one_static: n_embd above 4096 or n_ffn above 16384 exceeds the built-in scratch; "
+                                   "use frhip_ffn_one with a workspace");
+  void* ws = nullptr;
+  FR_TRY(static_scratch(&ws));
+  // r [C] and relu(k)^2 [F] are written in full by the first launch before the second reads them:
+  // nothing in the scratch has to start at zero, whatever an earlier (larger) call left there.
+  return frhip_ffn_one(C, F, x, sx, ln_w, ln_b, k_mix, r_mix, kw, vw, rw, x_out, xx_out, post_div2, ws, s);
 }
 
 extern "C" int frhip_head(int C, const void* x, const void* ln_w, const void* ln_b, const frhip_weight* head,

@@ -18,5 +18,7 @@ int check_launch(const char* kernel);
 // workgroup per CU most decode launches are a single register-resident batch per wave).
 int decode_grid();
 int compute_units();
+// Device address of the current device's built-in decode scratch (looked up once per device).
+int static_scratch(void** ptr);
 
 }  // namespace frhip

@@ -84,7 +84,7 @@ int frhip_init(int device) {
   }
   g_cus = 0;
   compute_units();
-  return 0;
+  return static_scratch(nullptr);  // this device's copy of the built-in scratch
 }
 
 int frhip_device_info(char* name, size_t name_len, int* cus, size_t* total_mem) {

@@ -147,6 +147,19 @@ int frhip_ffn_one(int C, int F, const void *x, const void *sx, const void *ln_w,
                   const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
                   void *x_out, void *xx_out, int post_div2, void *workspace, frhip_stream s);
 
+/* frhip_ffn_one without a workspace argument and without any allocation.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory or hand over a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The
+ * intermediate vectors (sigmoid(r) [C], relu(k)^2 [F]) live in a 112 KB device array built into the
+ * library, one copy per GPU, held until the process ends.  Limits: C <= 4096, F <= 16384, else
+ * FRHIP_ESHAPE.  All calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered.  Results are those of
+ * frhip_ffn_one bit for bit. */
+int frhip_ffn_one_static(int C, int F, const void *x, const void *sx, const void *ln_w, const void *ln_b,
+                         const void *k_mix, const void *r_mix,
+                         const frhip_weight *kw, const frhip_weight *vw, const frhip_weight *rw,
+                         void *x_out, void *xx_out, int post_div2, frhip_stream s);
+
 /* layernorm(ln_out) -> head matmul -> cast to fp32: kernels/default/model_forward.cpp:180-188. */
 int frhip_head(int C, const void *x, const void *ln_w, const void *ln_b, const frhip_weight *head, float *logits, frhip_stream s);
 /* The same with a second destination: every logit is also stored to mirror [N] (fp32), meant for pinned host
