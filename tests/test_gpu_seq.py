@@ -109,8 +109,6 @@ def _common(C_):
 @pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1024, 2048, 8192), (512, 2560, 8960), (1, 512, 1024), (33, 768, 3072)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_ffn_seq(T, C_, F_, quant):
-    if quant and C_ >= 2048:
-        pytest.skip("covered by the fp16 case at this size; uint8 covered at the smaller sizes")
     g = np.random.default_rng(5000 + T) if T >= 512 else rng  # the full-size cases draw from a stream of their own
     x, sx = h(g.standard_normal((T, C_)) * 2), h(g.standard_normal(C_))
     ln_w, ln_b = h(1 + 0.1 * g.standard_normal(C_)), h(0.1 * g.standard_normal(C_))
@@ -138,8 +136,6 @@ def _state_v4(C_, fresh):
 @pytest.mark.parametrize("quant", [False, True])
 @pytest.mark.parametrize("fresh", [True, False])
 def test_att_seq_v4(T, C_, quant, fresh):
-    if C_ == 2048 and (quant or not fresh):
-        pytest.skip("full-size case runs once")
     x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
     aa, bb, pp = _state_v4(C_, fresh)
     ln_w, ln_b = _common(C_)
@@ -171,8 +167,6 @@ def test_att_seq_v4(T, C_, quant, fresh):
 @pytest.mark.parametrize("T,C_,H_", [(48, 512, 8), (512, 2560, 40), (1, 512, 8), (77, 512, 8)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_att_seq_v5_2(T, C_, H_, quant):
-    if C_ == 2560 and quant:
-        pytest.skip("full-size case runs once")
     S_ = C_ // H_
     x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
     s = rng.standard_normal((H_, S_, S_)).astype(np.float32)
@@ -204,8 +198,6 @@ def test_att_seq_v5_2(T, C_, H_, quant):
 @pytest.mark.parametrize("quant", [False, True])
 def test_att_seq_v5(T, C_, H_, quant):
     """RWKV-5.0 seq attention against the oracle's matrix form (kernels/cuda/att_seq.cu:158-256)."""
-    if C_ == 2048 and quant:
-        pytest.skip("full-size case runs once")
     S_ = C_ // H_
     x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
     s = rng.standard_normal((H_, S_, S_)).astype(np.float32)
