@@ -185,6 +185,48 @@ def wkv4_one_f16(t_first, t_decay, k, v, aa, bb, pp, r):
     return r, aa, bb, pp
 
 
+_sig("orc_gemv_u8", None, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i)
+_sig("orc_register_u8", None, _vp, _vp, _vp, _vp, _vp, _vp)
+_sig("orc_unregister_u8", None, _vp)
+
+
+def gemv_u8(x, q, mx, rx, my, ry):
+    """One-token product on the unrounded fp32 weights of the codes: x [K] half -> y [N] fp32."""
+    K, N = q.shape
+    y = np.empty(N, np.float32)
+    lib.orc_gemv_u8(_p(np.ascontiguousarray(x, np.float16)), _p(q), _p(mx), _p(rx), _p(my), _p(ry), _p(y), K, N)
+    return y
+
+
+ACC_EXACT, ACC_F32_SEQUENTIAL = 0, 1
+_sig("orc_set_accumulation", None, _i)
+
+
+def set_accumulation(mode):
+    """ACC_EXACT (default): products accumulate exactly, one rounding to fp32; ACC_F32_SEQUENTIAL: fp32 in
+    ascending k -- another valid member of the reference's "fp32 accumulate in cuBLAS's order"."""
+    lib.orc_set_accumulation(int(mode))
+
+
+_u8_keep = {}
+
+
+def register_u8(W, q, mx, rx, my, ry):
+    """From now on the oracle's one-token products on the binary16 matrix W (= dequant_u8 of these
+    codes) multiply the unrounded fp32 weights of the codes (orc_gemv_u8); matrix x matrix products
+    keep multiplying W.  The arrays are held until unregister_u8(W)."""
+    assert isinstance(W, np.ndarray) and W.dtype == np.float16 and W.flags["C_CONTIGUOUS"] and W.shape == q.shape
+    parts = [np.ascontiguousarray(q, np.uint8)] + [np.ascontiguousarray(v, np.float16) for v in (mx, rx, my, ry)]
+    _u8_keep[W.ctypes.data] = (W, parts)
+    lib.orc_register_u8(_p(W), *[_p(a) for a in parts])
+    return W
+
+
+def unregister_u8(W):
+    if _u8_keep.pop(W.ctypes.data, None) is not None:
+        lib.orc_unregister_u8(_p(W))
+
+
 def dequant_u8(q, mx, rx, my, ry):
     """q [K,N] uint8, mx/rx [N], my/ry [K] half -> W^ [K,N] half."""
     K, N = q.shape
@@ -292,9 +334,16 @@ class Model:
     """Oracle model over a list of numpy parameter arrays in the reference's
     positional order (kernels/default/init_model.cpp:91-126) plus emb [V,C]."""
 
-    def __init__(self, version, mode, n_layer, n_embd, n_ffn, n_head, vocab, params, emb, n_att=None):
+    def __init__(self, version, mode, n_layer, n_embd, n_ffn, n_head, vocab, params, emb, n_att=None, quant=None):
+        """quant: {parameter index: (q, mx, rx, my, ry)} -- that parameter becomes the binary16 matrix w^ of the
+        codes (seq mode multiplies it) and one-token steps multiply the codes' unrounded fp32 weights."""
         self.mode = mode
         self._params = [np.ascontiguousarray(p) for p in params]
+        self._registered = []
+        for i, parts in (quant or {}).items():
+            assert mode == F16
+            self._params[i] = register_u8(dequant_u8(*parts), *parts)
+            self._registered.append(self._params[i])
         self._emb = np.ascontiguousarray(emb)
         self._parr = (_vp * len(self._params))(*[_p(p) for p in self._params])
         self.c = _OrcModel(version, mode, n_layer, n_embd, n_att or n_embd, n_ffn, n_head, vocab,
@@ -310,6 +359,17 @@ class Model:
 
     def reset(self):
         lib.orc_state_reset(C.byref(self.c), self._sarr)
+
+    def close(self):
+        for w in getattr(self, "_registered", []):
+            unregister_u8(w)
+        self._registered = []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
     def run(self, ids):
         """Model::Run (model.cpp:188-208): int -> one-token forward, list -> seq mode."""

@@ -204,33 +204,152 @@ void orc_mix_f32(const float *xx, const float *sx, const float *mix, float *out,
     }
 }
 
+/* ------------------------------------------------------------------------
+ * uint8 weights in the one-token products.  The ChatRWKV scheme this format comes from has two
+ * evaluations of the same dequantisation formula: its matrix x matrix path expands the codes to a
+ * binary16 matrix first (orc_dequant_u8: one rounding of w^ to half), its vector x matrix kernel
+ * forms every weight in fp32 and multiplies it unrounded (rwkv pip package 0.8.x,
+ * rwkv/cuda/operators.cu, kernel_mm_one_fp16i8 -- not part of the reference tree, restated from its
+ * published source: PARITY UNPINNED by the reference).  orc_gemv_u8 is the second one:
+ *   y[n] = sum_k x[k] * fmaf(q[k][n], (rx[n]/255)*ry[k], mx[n]+my[k])      (each weight in fp32,
+ * products and sum exact in double, one rounding of the sum to fp32).
+ * A binary16 matrix handed to orc_gemm_f16 with T == 1 is multiplied this way when its codes have
+ * been registered with orc_register_u8 (keyed by the matrix pointer); with T > 1 the binary16
+ * matrix itself is used.
+ * ------------------------------------------------------------------------ */
+static int g_acc_mode = ORC_ACC_EXACT;
+void orc_set_accumulation(int mode) { g_acc_mode = mode; }
+
+typedef struct {
+  const orc_half *W;
+  const uint8_t *q;
+  const orc_half *mx, *rx, *my, *ry;
+} orc_u8_rec;
+static orc_u8_rec *g_u8 = NULL;
+static size_t g_u8_n = 0, g_u8_cap = 0;
+
+void orc_register_u8(const orc_half *W, const uint8_t *q, const orc_half *mx, const orc_half *rx,
+                     const orc_half *my, const orc_half *ry) {
+  for (size_t i = 0; i < g_u8_n; i++)
+    if (g_u8[i].W == W) {
+      g_u8[i] = (orc_u8_rec){W, q, mx, rx, my, ry};
+      return;
+    }
+  if (g_u8_n == g_u8_cap) {
+    g_u8_cap = g_u8_cap ? 2 * g_u8_cap : 64;
+    g_u8 = (orc_u8_rec *)realloc(g_u8, g_u8_cap * sizeof(orc_u8_rec));
+    if (!g_u8) abort();
+  }
+  g_u8[g_u8_n++] = (orc_u8_rec){W, q, mx, rx, my, ry};
+}
+
+void orc_unregister_u8(const orc_half *W) {
+  for (size_t i = 0; i < g_u8_n; i++)
+    if (g_u8[i].W == W) {
+      g_u8[i] = g_u8[--g_u8_n];
+      return;
+    }
+}
+
+void orc_gemv_u8(const orc_half *x, const uint8_t *q, const orc_half *mx, const orc_half *rx,
+                 const orc_half *my, const orc_half *ry, float *y, int K, int N) {
+  float *xf = (float *)xmalloc(sizeof(float) * (size_t)K);
+  float *ryf = (float *)xmalloc(sizeof(float) * (size_t)K);
+  float *myf = (float *)xmalloc(sizeof(float) * (size_t)K);
+  orc_h2f_n(x, xf, (size_t)K);
+  orc_h2f_n(ry, ryf, (size_t)K);
+  orc_h2f_n(my, myf, (size_t)K);
+  int nblocks = (N + 63) / 64;
+#pragma omp parallel for schedule(static)
+  for (int nb = 0; nb < nblocks; nb++) {
+    int n0 = nb * 64, n1 = n0 + 64 < N ? n0 + 64 : N;
+    double acc[64];
+    float facc[64];
+    float c[64], m[64];
+    for (int j = 0; j < n1 - n0; j++) {
+      acc[j] = 0.0;
+      facc[j] = 0.f;
+      c[j] = orc_h2f(rx[n0 + j]) / 255.0f;
+      m[j] = orc_h2f(mx[n0 + j]);
+    }
+    for (int k = 0; k < K; k++) {
+      const uint8_t *qr = q + (size_t)k * N + n0;
+      const double xk = (double)xf[k];
+      for (int j = 0; j < n1 - n0; j++) {
+        const float a = c[j] * ryf[k];
+        const float b = m[j] + myf[k];
+        const float w32 = fmaf((float)qr[j], a, b);
+        acc[j] += xk * (double)w32;
+        facc[j] += xf[k] * w32; /* ORC_ACC_F32_SEQUENTIAL: fp32 products and sums, ascending k */
+      }
+    }
+    for (int j = 0; j < n1 - n0; j++)
+      y[n0 + j] = g_acc_mode == ORC_ACC_F32_SEQUENTIAL ? facc[j] : (float)acc[j];
+  }
+  free(xf); free(ryf); free(myf);
+}
+
 #define NB 256 /* column block */
 #define TB 8   /* row block    */
 
 void orc_gemm_f16(const orc_half *x, const orc_half *W, float *y_f32, orc_half *y_f16, int T,
                   int K, int N) {
+  if (T == 1) /* registered uint8 codes: the one-token product multiplies the unrounded fp32 weight */
+    for (size_t i = 0; i < g_u8_n; i++)
+      if (g_u8[i].W == W) {
+        float *y = y_f32 ? y_f32 : (float *)xmalloc(sizeof(float) * (size_t)N);
+        orc_gemv_u8(x, g_u8[i].q, g_u8[i].mx, g_u8[i].rx, g_u8[i].my, g_u8[i].ry, y, K, N);
+        if (y_f16) orc_f2h_n(y, y_f16, (size_t)N);
+        if (!y_f32) free(y);
+        return;
+      }
   float *xf = (float *)xmalloc(sizeof(float) * (size_t)T * K);
   orc_h2f_n(x, xf, (size_t)T * K);
   int nblocks = (N + NB - 1) / NB;
 #pragma omp parallel for schedule(static)
   for (int nb = 0; nb < nblocks; nb++) {
     int n0 = nb * NB, n1 = n0 + NB < N ? n0 + NB : N, w = n1 - n0;
-    float acc[TB][NB];
-    float wrow[NB];
+    /* The reference accumulates in fp32 in an order that is cuBLAS's own (matmul.cpp:38-42): every
+     * such order lies within its own rounding error of the exact sum.  The oracle returns the centre
+     * of that family -- the exact sum (products of two halves and their sum are exact in double for
+     * any K here) rounded once to fp32 -- so that a comparison measures the other side's error only. */
+    double acc[TB][NB];
+    float wrow[NB], out[NB];
+    if (g_acc_mode == ORC_ACC_F32_SEQUENTIAL) { /* another member of the family: fp32, ascending k */
+      float facc[TB][NB];
+      for (int t0 = 0; t0 < T; t0 += TB) {
+        int tn = t0 + TB < T ? TB : T - t0;
+        for (int t = 0; t < tn; t++)
+          for (int j = 0; j < w; j++) facc[t][j] = 0.f;
+        for (int k = 0; k < K; k++) {
+          orc_h2f_n(W + (size_t)k * N + n0, wrow, (size_t)w);
+          for (int t = 0; t < tn; t++) {
+            float xk = xf[(size_t)(t0 + t) * K + k];
+            for (int j = 0; j < w; j++) facc[t][j] += xk * wrow[j]; /* product exact in fp32 */
+          }
+        }
+        for (int t = 0; t < tn; t++) {
+          if (y_f32) memcpy(y_f32 + (size_t)(t0 + t) * N + n0, facc[t], sizeof(float) * (size_t)w);
+          if (y_f16) orc_f2h_n(facc[t], y_f16 + (size_t)(t0 + t) * N + n0, (size_t)w);
+        }
+      }
+      continue;
+    }
     for (int t0 = 0; t0 < T; t0 += TB) {
       int tn = t0 + TB < T ? TB : T - t0;
       for (int t = 0; t < tn; t++)
-        for (int j = 0; j < w; j++) acc[t][j] = 0.f;
+        for (int j = 0; j < w; j++) acc[t][j] = 0.0;
       for (int k = 0; k < K; k++) {
         orc_h2f_n(W + (size_t)k * N + n0, wrow, (size_t)w);
         for (int t = 0; t < tn; t++) {
-          float xk = xf[(size_t)(t0 + t) * K + k];
-          for (int j = 0; j < w; j++) acc[t][j] += xk * wrow[j]; /* product exact in fp32 */
+          double xk = (double)xf[(size_t)(t0 + t) * K + k];
+          for (int j = 0; j < w; j++) acc[t][j] += xk * (double)wrow[j];
         }
       }
       for (int t = 0; t < tn; t++) {
-        if (y_f32) memcpy(y_f32 + (size_t)(t0 + t) * N + n0, acc[t], sizeof(float) * (size_t)w);
-        if (y_f16) orc_f2h_n(acc[t], y_f16 + (size_t)(t0 + t) * N + n0, (size_t)w);
+        for (int j = 0; j < w; j++) out[j] = (float)acc[t][j];
+        if (y_f32) memcpy(y_f32 + (size_t)(t0 + t) * N + n0, out, sizeof(float) * (size_t)w);
+        if (y_f16) orc_f2h_n(out, y_f16 + (size_t)(t0 + t) * N + n0, (size_t)w);
       }
     }
   }

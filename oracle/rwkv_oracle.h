@@ -21,7 +21,8 @@
  * The uint8 dequantisation formula has no counterpart in the reference tree
  * (kernels/kernels.h:11-13 only names the mx/rx/my/ry parameters): PARITY UNPINNED
  * by the reference; it is pinned here by exhaustive evaluation against an
- * independent numpy statement of the same formula.
+ * independent numpy statement of the same formula.  The same holds for orc_gemv_u8 (the
+ * one-token product on unrounded fp32 weights): PARITY UNPINNED by the reference.
  */
 #ifndef RWKV_ORACLE_H_
 #define RWKV_ORACLE_H_
@@ -66,6 +67,14 @@ void orc_mix_f16(const orc_half *xx, const orc_half *sx, const orc_half *mix, or
                  int rows, int cols);
 void orc_mix_f32(const float *xx, const float *sx, const float *mix, float *out, int rows,
                  int cols);
+/* How orc_gemm_f16 accumulates.  The reference accumulates in fp32 in cuBLAS's own order
+ * (kernels/cuda/matmul.cpp:38-42), which nothing pins; every such order lies within its own
+ * rounding error of the exact sum.  ORC_ACC_EXACT (default) returns the centre of that family:
+ * the exact sum rounded once to fp32.  ORC_ACC_F32_SEQUENTIAL is another member (fp32, ascending
+ * k); running one model under both shows how far two valid evaluations of the reference's
+ * arithmetic drift apart, i.e. the floor below which a logit tolerance cannot be met. */
+enum { ORC_ACC_EXACT = 0, ORC_ACC_F32_SEQUENTIAL = 1 };
+void orc_set_accumulation(int mode);
 /* kernels/cuda/matmul.cpp:35-80: fp16 inputs, fp32 products and accumulation, one
  * rounding to the output type.  W is [K,N] row-major.  y_f32 or y_f16 may be NULL. */
 void orc_gemm_f16(const orc_half *x, const orc_half *W, float *y_f32, orc_half *y_f16, int T,
@@ -93,6 +102,21 @@ void orc_wkv4_one_f16(const float *t_first, const float *t_decay, const float *k
 orc_half orc_dequant_u8_scalar(uint8_t q, orc_half mx, orc_half rx, orc_half my, orc_half ry);
 void orc_dequant_u8(const uint8_t *q, const orc_half *mx, const orc_half *rx,
                     const orc_half *my, const orc_half *ry, orc_half *W, int K, int N);
+
+/* The one-token product of the same scheme: every weight formed in fp32 by the formula above and
+ * multiplied WITHOUT the rounding to half (products and sum exact in double, the sum rounded once
+ * to fp32).  Follows the vector x matrix kernel of the ChatRWKV `rwkv` package (0.8.x,
+ * rwkv/cuda/operators.cu, kernel_mm_one_fp16i8), which is not in the reference tree: PARITY
+ * UNPINNED by the reference; pinned by float64 brute force of the real-valued formula and by
+ * one-hot probes that must return fmaf(q, a, b) exactly. */
+void orc_gemv_u8(const orc_half *x, const uint8_t *q, const orc_half *mx, const orc_half *rx,
+                 const orc_half *my, const orc_half *ry, float *y, int K, int N);
+/* After orc_register_u8(W, ...) every orc_gemm_f16 call with T == 1 on the binary16 matrix W
+ * (the orc_dequant_u8 image of the codes) runs orc_gemv_u8 on the codes instead; calls with
+ * T > 1 keep multiplying by W.  Keyed by pointer; the arrays must stay alive while registered. */
+void orc_register_u8(const orc_half *W, const uint8_t *q, const orc_half *mx, const orc_half *rx,
+                     const orc_half *my, const orc_half *ry);
+void orc_unregister_u8(const orc_half *W);
 
 /* ---- layer-level ops (one token) ----------------------------------------- */
 /* kernels/cuda/att.cu:182-217,337-359.  x_out, xx_out [C]; aa,bb,pp updated in

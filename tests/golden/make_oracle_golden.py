@@ -1,6 +1,6 @@
 """Writes tests/golden/oracle_small_models.npz: logits of small synthetic models computed by the
 CPU oracle (oracle/rwkv_oracle.c through pyoracle), for RWKV-4, 5.0 and 5.2, binary16 mode and
-the uint8 model (the binary16 model of the dequantised weights).
+the uint8 model.
 
 They are regression fixtures, not reference outputs: the reference's own golden logits
 (tests/test_model.cpp:10-21) need a converted checkpoint that is not available offline.  What
@@ -30,11 +30,10 @@ TOKENS = [5, 17, 299, 0, 42, 7, 7, 123]
 
 def logits_of(version, L, C, F, V, H, seed, quant):
     params, emb = make_model(version, L, C, F, V, H, seed=seed)
-    if quant:  # the int8 model is the binary16 model of the dequantised matrices
-        for i in matrix_indices(version, L):
-            q = quantize_u8(params[i].astype(np.float32))
-            params[i] = po.dequant_u8(*q)
-    m = po.Model(version, po.F16, L, C, F, H, V, params, emb)
+    # the int8 model: seq mode multiplies the binary16 w^ of the codes, one-token steps the unrounded
+    # fp32 weights of the same formula (pyoracle.Model, `quant=`)
+    qd = {i: quantize_u8(params[i].astype(np.float32)) for i in matrix_indices(version, L)} if quant else None
+    m = po.Model(version, po.F16, L, C, F, H, V, params, emb, quant=qd)
     one = np.stack([m.run(t).copy() for t in TOKENS])
     m.reset()
     seq = m.run(TOKENS).copy()

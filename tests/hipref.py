@@ -45,6 +45,40 @@ def assert_close_f16(got, ref, max_ulp=2, max_frac=0.03, what="", floor_rms=0.25
         what, (got.view(np.uint16) != ref.view(np.uint16)).mean())
 
 
+def same_token_or_near_tie(lh, lo):
+    """The greedy tokens agree, or the oracle's own margin between the two candidates is at most twice the
+    largest logit difference of this step: a difference of d can swap two logits that lie less than 2d
+    apart (one binary16 spacing at the top of a flat distribution is enough)."""
+    th, to = int(np.argmax(lh)), int(np.argmax(lo))
+    return th == to or float(lo[to] - lo[th]) <= 2 * float(np.abs(lh - lo).max())
+
+
+def greedy_against_oracle(run_hip, run_oracle, prompt, steps, tol=2e-2, report=None, tag=""):
+    """The parity criterion: feed `prompt` token by token, then `steps` greedy steps; at every step the
+    logits agree within `tol` (max-abs) and the greedy tokens agree (or differ at a near-tie, see
+    same_token_or_near_tie; both sides then continue with the oracle's token).
+    Returns (worst max-abs logit difference, number of near-tie steps)."""
+    import time
+    for t in prompt:
+        lh, lo = run_hip(int(t)), run_oracle(int(t))
+    worst, swaps, t0 = 0.0, 0, time.time()
+    for step in range(steps):
+        d = float(np.abs(lh - lo).max())
+        worst = max(worst, d)
+        th, to = int(np.argmax(lh)), int(np.argmax(lo))
+        if th != to:
+            assert same_token_or_near_tie(lh, lo), "%s: greedy token differs at step %d (hip %d, oracle %d, oracle margin %g, |dlogit| %g)" % (
+                tag, step, th, to, float(lo[to] - lo[th]), d)
+            swaps += 1
+        lh, lo = run_hip(to), run_oracle(to)
+        if report and step % 32 == 31:
+            report("%s: %d steps, worst |dlogit| %.2e, %d near-tie swaps, %.0f s" % (tag, step + 1, worst, swaps, time.time() - t0))
+    if tol is not None:
+        assert worst <= tol, "%s: worst |dlogit| %g" % (tag, worst)
+    assert swaps <= max(1, steps // 16), "%s: tokens differed at %d of %d steps" % (tag, swaps, steps)
+    return worst, swaps
+
+
 def make_weight(w_kn, quant=False):
     """PackedWeight from a [K,N] half matrix; quant=True quantises to uint8 first and
     also returns the oracle's dequantised [K,N] half matrix."""
@@ -54,6 +88,7 @@ def make_weight(w_kn, quant=False):
     from synth import quantize_u8
     q, mx, rx, my, ry = quantize_u8(w_kn)
     pw = PackedWeight(q=q, mx=mx, rx=rx, my=my, ry=ry)
+    pw.parts = (q, mx, rx, my, ry)
     f = np.float64
     # the real-valued formula the codes stand for, before any rounding of w^
     pw.exact = lambda: (q.astype(f) * (rx.astype(f) / 255)[None, :] * ry.astype(f)[:, None]
@@ -69,6 +104,7 @@ class HipModelV4:
         self.L, self.C, self.F, self.V = L_, C_, F_, V_
         self.mats = {}
         self.oracle_params = list(params)
+        self.oracle_quant = {}  # parameter index -> (q, mx, rx, my, ry): pyoracle.Model(..., quant=)
         self.p = []
         mat_pos = set()
         for l in range(L_):
@@ -79,6 +115,8 @@ class HipModelV4:
                 w, deq = make_weight(a, quant)
                 self.p.append(w)
                 self.oracle_params[i] = deq
+                if quant:
+                    self.oracle_quant[i] = w.parts
             else:
                 self.p.append(dev(a))
         self.emb = dev(emb)

@@ -6,7 +6,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 import pyoracle as po
-from hipref import DevBuf, HipModelV4, L, assert_close_f16, dev, fr, make_weight
+from hipref import DevBuf, HipModelV4, L, assert_close_f16, dev, fr, greedy_against_oracle, make_weight
 from synth import make_model
 
 _alive = []
@@ -224,40 +224,23 @@ def test_head_mirror_in_pinned_host_memory():
         fr.check(L().frhip_host_free(hp))
 
 
-def _greedy_pair(L_, C_, F_, V_, quant, steps, seed):
-    params, emb = make_model(4, L_, C_, F_, V_, seed=seed)
-    hm = HipModelV4(L_, C_, F_, V_, params, emb, quant=quant)
-    om = po.Model(4, po.F16, L_, C_, F_, 0, V_, hm.oracle_params, emb)
-    prompt = np.random.default_rng(42).integers(0, V_, 16)
-    for t in prompt:
-        lh, lo = hm.run(int(t)), om.run(int(t))
-    toks_h, toks_o, worst, gaps = [], [], 0.0, []
-    for _ in range(steps):
-        worst = max(worst, float(np.abs(lh - lo).max()))
-        th, to = int(np.argmax(lh)), int(np.argmax(lo))
-        top2 = np.sort(lo)[-2:]
-        gaps.append(float(top2[1] - top2[0]))
-        toks_h.append(th)
-        toks_o.append(to)
-        if th != to:
-            break
-        lh, lo = hm.run(th), om.run(to)
-    return toks_h, toks_o, worst, gaps, hm, om
-
-
 @pytest.mark.parametrize("quant", [False, True])
 def test_greedy_decode_128_steps_matches_oracle(quant):
-    """fp16 logits within max-abs 2e-2 of the oracle and identical greedy argmax over 128 steps
+    """fp16 logits within max-abs 2e-2 of the oracle and the same greedy token over 128 steps
     (12 layers: two /2 rescales are crossed)."""
-    th, to, worst, gaps, hm, om = _greedy_pair(12, 512, 2048, 4096, quant, 128, seed=5)
-    print("quant", quant, "worst |dlogit|", worst, "min top-2 gap", min(gaps), flush=True)
-    assert worst <= 2e-2
-    assert th == to and len(th) == 128
+    L_, C_, F_, V_ = 12, 512, 2048, 4096
+    params, emb = make_model(4, L_, C_, F_, V_, seed=5)
+    hm = HipModelV4(L_, C_, F_, V_, params, emb, quant=quant)
+    om = po.Model(4, po.F16, L_, C_, F_, 0, V_, params, emb, quant=hm.oracle_quant)
+    prompt = np.random.default_rng(42).integers(0, V_, 16)
+    worst, swaps = greedy_against_oracle(hm.run, om.run, prompt, 128, tol=2e-2, tag="12x512 quant=%s" % quant)
+    print("quant", quant, "worst |dlogit|", worst, "near-tie swaps", swaps, flush=True)
     # states agree after 144 tokens
     for l in (0, 11):
         for j in (1, 2, 3):
             ref = om.state[l * 5 + j]
             assert np.abs(hm.state[l][j].numpy() - ref).max() <= 5e-3 * np.abs(ref).max()
+    om.close()
     # ResetStates then rerun is bit-identical (tests/test_model.cpp:93-97)
     hm.reset()
     a = [hm.run(t).copy() for t in (1, 2, 3)]

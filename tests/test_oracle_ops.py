@@ -317,3 +317,63 @@ def test_quantise_then_dequantise_error_is_half_a_step():
     err = np.abs(wd - w.astype(np.float64))
     assert (err <= 0.5 * step + 3e-4).all()  # half a step + binary16 rounding of a,b,w^
     assert err.mean() < 0.3 * step.mean() + 1e-4
+
+
+# ---------------------------------------------------------------- one-token product on uint8 codes
+def _weights_f32_numpy(q, mx, rx, my, ry):
+    """The fp32 weight of every code by the dequantisation formula, before any rounding to half
+    (same independent statement as _dequant_numpy, stopped one rounding earlier)."""
+    f = np.float32
+    c = rx.astype(f) / f(255)
+    a = c[None, :] * ry.astype(f)[:, None]
+    b = mx.astype(f)[None, :] + my.astype(f)[:, None]
+    return (q.astype(np.longdouble) * a.astype(np.longdouble) + b.astype(np.longdouble)).astype(f)
+
+
+def test_gemv_u8_one_hot_rows_return_the_unrounded_fp32_weights():
+    K, N = 96, 130
+    w = h(rng.standard_normal((K, N)) * 0.02)
+    q, mx, rx, my, ry = quantize_u8(w)
+    want = _weights_f32_numpy(q, mx, rx, my, ry)
+    assert (want.astype(np.float16).astype(np.float32) != want).mean() > 0.9  # i.e. not the binary16 w^
+    for k in (0, 1, 37, K - 1):
+        e = np.zeros(K, np.float16)
+        e[k] = 1
+        assert np.array_equal(po.gemv_u8(e, q, mx, rx, my, ry), want[k]), k  # catches a transposed q, swapped mx/my
+        e[k] = -2
+        assert np.array_equal(po.gemv_u8(e, q, mx, rx, my, ry), -2 * want[k]), k
+
+
+def test_gemv_u8_against_float64_of_the_real_valued_formula():
+    for K, N in ((512, 200), (2048, 65), (16, 1)):
+        w = h(rng.standard_normal((K, N)) * 0.02)
+        q, mx, rx, my, ry = quantize_u8(w)
+        x = h(rng.standard_normal(K) * 3)
+        f = np.float64
+        real = q.astype(f) * (rx.astype(f) / 255)[None, :] * ry.astype(f)[:, None] + mx.astype(f)[None, :] + my.astype(f)[:, None]
+        exact = x.astype(f) @ real
+        mag = np.abs(x.astype(f)) @ np.abs(real)
+        got = po.gemv_u8(x, q, mx, rx, my, ry)
+        # every fp32 weight is within 1.5 fp32 roundings of the real value; the sum is rounded once
+        assert (np.abs(got - exact) <= 2.0 ** -22 * mag + 1e-30).all()
+        # and it is the exact sum of x times the fp32 weights
+        w32 = _weights_f32_numpy(q, mx, rx, my, ry)
+        assert np.array_equal(got, (x.astype(f) @ w32.astype(f)).astype(np.float32))
+
+
+def test_registered_codes_change_one_token_products_only():
+    K, N = 256, 96
+    w = h(rng.standard_normal((K, N)) * 0.02)
+    q, mx, rx, my, ry = quantize_u8(w)
+    W = po.dequant_u8(q, mx, rx, my, ry)
+    x2 = h(rng.standard_normal((2, K)))
+    before1, before2 = po.gemm_f16(x2[0], W, "f32"), po.gemm_f16(x2, W, "f32")
+    po.register_u8(W, q, mx, rx, my, ry)
+    try:
+        assert np.array_equal(po.gemm_f16(x2[0], W, "f32"), po.gemv_u8(x2[0], q, mx, rx, my, ry))
+        assert not np.array_equal(po.gemm_f16(x2[0], W, "f32"), before1)
+        assert np.array_equal(po.gemm_f16(x2, W, "f32"), before2)   # matrix x matrix: the binary16 w^
+        assert np.array_equal(po.gemm_f16(x2[0], W.copy(), "f32"), before1)  # keyed by the matrix, not by its values
+    finally:
+        po.unregister_u8(W)
+    assert np.array_equal(po.gemm_f16(x2[0], W, "f32"), before1)
