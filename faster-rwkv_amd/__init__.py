@@ -81,6 +81,10 @@ _SIGS = {
     "frhip_fill": (_i, [_vp, _i, C.c_float, _sz, _vp]),
     "frhip_scalar_div_f16": (_i, [_vp, C.c_float, _sz, _vp]),
     "frhip_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "frhip_slice": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "frhip_cat": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _i, _vp]),
+    "frhip_transpose": (_i, [_vp, _vp, _i, _vp, _i, _i, _i, _vp]),
+    "frhip_silu": (_i, [_vp, _vp, _i, _sz, _vp]),
     "frhip_embed_ring": (_i, [_vp, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "frhip_decode_workspace_bytes": (_sz, [_i, _i]),
     "frhip_att_one_v4": (_i, [_i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),
@@ -257,12 +261,49 @@ def host():
         h.fr_model_save_state.argtypes = [_vp, C.c_char_p]
         h.fr_model_load_state.argtypes = [_vp, C.c_char_p]
         h.fr_model_get_state.argtypes = [_vp, _i, _i, _vp, _i]
+        h.fr_model_snapshot.restype = _vp
+        h.fr_model_snapshot.argtypes = [_vp]
+        h.fr_model_restore.argtypes = [_vp, _vp]
+        h.fr_snapshot_free.argtypes = [_vp]
         h.fr_greedy_decode.restype = C.c_longlong
         h.fr_greedy_decode.argtypes = [_vp, _i, _i, _vp]
         h.fr_quantize_u8.argtypes = [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp]
         h.fr_allocator_stats.argtypes = [C.POINTER(_sz)] * 3
+        h.fr_allocator_trim.restype = C.c_longlong
+        h.fr_hip_alloc.restype = _vp
+        h.fr_hip_alloc.argtypes = [_sz]
+        h.fr_hip_free.argtypes = [_vp]
+        h.fr_hip_shape_op.restype = C.c_longlong
+        h.fr_hip_shape_op.argtypes = [_i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, C.c_longlong, _vp, _vp]
         _host = h
     return _host
+
+
+def allocator_stats():
+    """(bytes reserved from the driver, bytes handed out, driver allocation calls so far) of the hip allocator."""
+    a, b, c = _sz(), _sz(), _sz()
+    if host().fr_allocator_stats(C.byref(a), C.byref(b), C.byref(c)) < 0:
+        raise FrhipError(host().fr_last_error().decode())
+    return a.value, b.value, c.value
+
+
+def shape_op(op, a, b=None, params=()):
+    """One registry call of slice (op 0), cat (1), transpose (2) or silu (3) on the hip device."""
+    a = np.ascontiguousarray(a)
+    code = {np.dtype(np.float32): 0, np.dtype(np.float16): 1, np.dtype(np.int8): 2}[a.dtype]
+    ash = (C.c_int * a.ndim)(*a.shape)
+    bsh = None
+    if b is not None:
+        b = np.ascontiguousarray(b, a.dtype)
+        bsh = (C.c_int * b.ndim)(*b.shape)
+    par = (C.c_int * max(len(params), 1))(*params)
+    out = np.empty(a.size + (b.size if b is not None else 0), a.dtype)
+    osh, ond = (C.c_int * 4)(), C.c_int()
+    n = host().fr_hip_shape_op(op, code, a.ctypes.data, ash, a.ndim, b.ctypes.data if b is not None else None, bsh, par,
+                               out.ctypes.data, out.nbytes, osh, C.byref(ond))
+    if n < 0:
+        raise FrhipError(host().fr_last_error().decode())
+    return out[:n].reshape([osh[i] for i in range(ond.value)])
 
 
 class Model:
@@ -311,6 +352,20 @@ class Model:
         buf = np.empty(1 << 22, np.uint8)
         n = self._chk(self._h.fr_model_get_state(self._m, layer, index, buf.ctypes.data, buf.size))
         return buf[:n].view(dtype).copy()
+
+    def snapshot(self):
+        """A copy of Model::states() (shares storage, as `auto s = model.states();` does); give it to restore()."""
+        s = self._h.fr_model_snapshot(self._m)
+        if not s:
+            raise FrhipError(self._h.fr_last_error().decode())
+        return s
+
+    def restore(self, snap):
+        """Model::set_states(snapshot)."""
+        self._chk(self._h.fr_model_restore(self._m, snap))
+
+    def free_snapshot(self, snap):
+        self._h.fr_snapshot_free(snap)
 
     def generate(self, sampler, first_id, steps, temperature=1.0, top_k=0, top_p=1.0):
         """chat.cpp:56-92 without its penalties, in C++; returns (token ids, seconds)."""

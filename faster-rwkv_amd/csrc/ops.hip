@@ -342,11 +342,102 @@ int dequant_u8_group_async(int nseg, const unsigned char* const* q, const h1* co
   return check_launch("dequant_u8 (group)");
 }
 
+// ---- shape operators (kernels/cuda/slice.cu:17-36, cat.cu:28-52, transpose.cu:16-34) ----------
+// Index math over at most four dimensions with the shapes passed by value: no device allocation
+// and no blocking copy per call.
+struct Dims4 {
+  int n[4];
+};
+
+// dst[i0..i3] = src[start + i * interval] per dimension
+template <typename T>
+__global__ __launch_bounds__(256) void slice_kernel(const T* __restrict__ src, T* __restrict__ dst, Dims4 src_shape,
+                                                    Dims4 dst_shape, Dims4 start, Dims4 interval, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  size_t rem = i, off = 0, stride = 1;
+#pragma unroll
+  for (int d = 3; d >= 0; d--) {
+    const size_t idx = rem % (size_t)dst_shape.n[d];
+    rem /= (size_t)dst_shape.n[d];
+    off += ((size_t)start.n[d] + idx * (size_t)interval.n[d]) * stride;
+    stride *= (size_t)src_shape.n[d];
+  }
+  dst[i] = src[off];
+}
+
+// out [left][a_mid + b_mid][right] from a [left][a_mid][right] and b [left][b_mid][right]
+template <typename T>
+__global__ __launch_bounds__(256) void cat_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out,
+                                                  size_t a_mid, size_t b_mid, size_t right, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t r = i % right, m = (i / right) % (a_mid + b_mid), l = i / (right * (a_mid + b_mid));
+  out[i] = m < a_mid ? a[(l * a_mid + m) * right + r] : b[(l * b_mid + (m - a_mid)) * right + r];
+}
+
+// dst = src with dimensions dim_a and dim_b exchanged
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_nd_kernel(const T* __restrict__ src, T* __restrict__ dst, Dims4 src_shape,
+                                                           int dim_a, int dim_b, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  Dims4 ds = src_shape;
+  const int t = ds.n[dim_a];
+  ds.n[dim_a] = ds.n[dim_b];
+  ds.n[dim_b] = t;
+  int idx[4];
+  size_t rem = i;
+#pragma unroll
+  for (int d = 3; d >= 0; d--) {
+    idx[d] = (int)(rem % (size_t)ds.n[d]);
+    rem /= (size_t)ds.n[d];
+  }
+  const int u = idx[dim_a];
+  idx[dim_a] = idx[dim_b];
+  idx[dim_b] = u;
+  size_t off = 0;
+#pragma unroll
+  for (int d = 0; d < 4; d++) off = off * (size_t)src_shape.n[d] + (size_t)idx[d];
+  dst[i] = src[off];
+}
+
+// silu.  binary16 rounds as the fused attention path does (kernels/cuda/att.cu:145-152):
+// x / (1 + half(exp(-x))) in half.  (The reference's standalone operator, activations/silu.cu:19,28,
+// evaluates x / (1 - exp(x)), which is not SiLU; nothing on its CUDA path calls it.)
+__global__ void silu_f16_kernel(const h1* __restrict__ x, h1* __restrict__ y, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = silu_h(x[i]);
+}
+__global__ void silu_f32_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = x[i] / (1.0f + expf(-x[i]));
+}
+
 }  // namespace frhip
 
 using namespace frhip;
 
 static unsigned blocks_for(size_t n, unsigned per) { return (unsigned)((n + per - 1) / per); }
+
+namespace {
+// Right-align `ndim` values into four slots, filling the leading ones with `fill`.
+bool to_dims4(const int* v, int ndim, int fill, Dims4* out) {
+  if (ndim < 1 || ndim > 4 || !v) return false;
+  for (int d = 0; d < 4; d++) out->n[d] = fill;
+  for (int d = 0; d < ndim; d++) out->n[4 - ndim + d] = v[d];
+  return true;
+}
+template <typename F>
+int by_elem_bytes(int elem_bytes, F&& f) {
+  switch (elem_bytes) {
+    case 1: f(uint8_t{}); return 0;
+    case 2: f(uint16_t{}); return 0;
+    case 4: f(uint32_t{}); return 0;
+    default: return set_error(FRHIP_EINVAL, "shape operator: elem_bytes must be 1, 2 or 4");
+  }
+}
+}  // namespace
 
 extern "C" {
 
@@ -493,6 +584,77 @@ int frhip_argmax_f32(const float* logits, int n, int32_t* out_id, frhip_stream s
   if (n <= 0) return set_error(FRHIP_ESHAPE, "argmax: empty input");
   hipLaunchKernelGGL(argmax_f32_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(s), logits, n, out_id);
   return check_launch("argmax");
+}
+
+int frhip_slice(const void* src, void* dst, int ndim, const int* src_shape, const int* start, const int* interval,
+                const int* dst_shape, int elem_bytes, frhip_stream s) {
+  if (!src || !dst) return set_error(FRHIP_EINVAL, "slice: null pointer");
+  Dims4 ss, ds, st4, iv;
+  if (!to_dims4(src_shape, ndim, 1, &ss) || !to_dims4(dst_shape, ndim, 1, &ds) || !to_dims4(start, ndim, 0, &st4) ||
+      !to_dims4(interval, ndim, 1, &iv))
+    return set_error(FRHIP_ESHAPE, "slice: 1 to 4 dimensions");
+  size_t total = 1;
+  for (int d = 0; d < 4; d++) {
+    if (ss.n[d] <= 0 || ds.n[d] < 0 || st4.n[d] < 0 || iv.n[d] <= 0) return set_error(FRHIP_ESHAPE, "slice: bad range");
+    if (ds.n[d] > 0 && (long)st4.n[d] + (long)(ds.n[d] - 1) * iv.n[d] >= ss.n[d])
+      return set_error(FRHIP_ESHAPE, "slice: range runs past the source dimension");
+    total *= (size_t)ds.n[d];
+  }
+  if (total == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(s);
+  int rc = by_elem_bytes(elem_bytes, [&](auto tag) {
+    using T = decltype(tag);
+    hipLaunchKernelGGL(slice_kernel<T>, dim3(blocks_for(total, 256)), dim3(256), 0, st, (const T*)src, (T*)dst, ss, ds, st4,
+                       iv, total);
+  });
+  return rc ? rc : check_launch("slice");
+}
+
+int frhip_cat(const void* a, const void* b, void* out, size_t left, size_t a_mid, size_t b_mid, size_t right,
+              int elem_bytes, frhip_stream s) {
+  if (!a || !b || !out) return set_error(FRHIP_EINVAL, "cat: null pointer");
+  const size_t total = left * (a_mid + b_mid) * right;
+  if (total == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(s);
+  int rc = by_elem_bytes(elem_bytes, [&](auto tag) {
+    using T = decltype(tag);
+    hipLaunchKernelGGL(cat_kernel<T>, dim3(blocks_for(total, 256)), dim3(256), 0, st, (const T*)a, (const T*)b, (T*)out,
+                       a_mid, b_mid, right, total);
+  });
+  return rc ? rc : check_launch("cat");
+}
+
+int frhip_transpose(const void* src, void* dst, int ndim, const int* shape, int dim_a, int dim_b, int elem_bytes,
+                    frhip_stream s) {
+  if (!src || !dst) return set_error(FRHIP_EINVAL, "transpose: null pointer");
+  Dims4 ss;
+  if (!to_dims4(shape, ndim, 1, &ss)) return set_error(FRHIP_ESHAPE, "transpose: 1 to 4 dimensions");
+  if (dim_a < 0 || dim_b < 0 || dim_a >= ndim || dim_b >= ndim) return set_error(FRHIP_EINVAL, "transpose: dimension out of range");
+  size_t total = 1;
+  for (int d = 0; d < 4; d++) {
+    if (ss.n[d] <= 0) return set_error(FRHIP_ESHAPE, "transpose: empty dimension");
+    total *= (size_t)ss.n[d];
+  }
+  hipStream_t st = static_cast<hipStream_t>(s);
+  int rc = by_elem_bytes(elem_bytes, [&](auto tag) {
+    using T = decltype(tag);
+    hipLaunchKernelGGL(transpose_nd_kernel<T>, dim3(blocks_for(total, 256)), dim3(256), 0, st, (const T*)src, (T*)dst, ss,
+                       dim_a + 4 - ndim, dim_b + 4 - ndim, total);
+  });
+  return rc ? rc : check_launch("transpose");
+}
+
+int frhip_silu(const void* x, void* y, int dtype, size_t n, frhip_stream s) {
+  if (!x || !y) return set_error(FRHIP_EINVAL, "silu: null pointer");
+  if (n == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(s);
+  if (dtype == FRHIP_F16)
+    hipLaunchKernelGGL(silu_f16_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, st, (const h1*)x, (h1*)y, n);
+  else if (dtype == FRHIP_F32)
+    hipLaunchKernelGGL(silu_f32_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, st, (const float*)x, (float*)y, n);
+  else
+    return set_error(FRHIP_EINVAL, "silu: dtype must be F16 or F32");
+  return check_launch("silu");
 }
 
 }  // extern "C"

@@ -104,7 +104,12 @@ int frhip_malloc(void** ptr, size_t bytes) {
   if (!ptr) return set_error(FRHIP_EINVAL, "ptr is null");
   *ptr = nullptr;
   if (bytes == 0) return 0;
-  HIP_TRY(hipMalloc(ptr, bytes));
+  const hipError_t e = hipMalloc(ptr, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // a refused allocation must not surface again as the next launch's error
+    *ptr = nullptr;
+    return hip_result(e, "hipMalloc");
+  }
   return 0;
 }
 

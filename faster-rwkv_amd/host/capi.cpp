@@ -14,6 +14,7 @@
 
 namespace rwkv::hip {
 void allocator_stats(size_t *reserved, size_t *in_use, size_t *driver_calls);
+size_t allocator_trim();
 }
 
 namespace {
@@ -163,6 +164,26 @@ int fr_model_load_state(void *m, const char *path) {
   });
 }
 
+// A snapshot as a C++ caller takes one: a copy of Model::states() (tensors that share storage with the
+// model's, no device copy), to be handed back through set_states() later.
+void *fr_model_snapshot(void *m) {
+  void *out = nullptr;
+  guarded([&]() {
+    out = new rwkv::States(static_cast<rwkv::Model *>(m)->states());
+    return 0;
+  });
+  return out;
+}
+
+int fr_model_restore(void *m, void *snapshot) {
+  return guarded([&]() {
+    static_cast<rwkv::Model *>(m)->set_states(*static_cast<rwkv::States *>(snapshot));
+    return 0;
+  });
+}
+
+void fr_snapshot_free(void *snapshot) { delete static_cast<rwkv::States *>(snapshot); }
+
 // Copy state tensor (layer, index) to the host as raw bytes; returns its size in bytes.
 int fr_model_get_state(void *m, int layer, int index, void *out, int capacity) {
   return guarded([&]() {
@@ -202,6 +223,68 @@ int fr_quantize_u8(const uint16_t *w_kn, int K, int N, uint8_t *q, uint16_t *mx,
                    uint16_t *ry) {
   return guarded([&]() {
     rwkv::hip::quantize_u8(w_kn, K, N, q, mx, rx, my, ry);
+    return 0;
+  });
+}
+
+// One call of a shape / activation operator through the registry on the `hip` device, on host data:
+// op 0 slice (params: start, interval, end per dimension), 1 cat (b, params[0] = dim), 2 transpose
+// (params: dim_a, dim_b), 3 silu.  dtype: 0 fp32, 1 fp16, 2 int8.  Writes the result and its shape;
+// returns the number of result elements.  For scripts and tests of the operator surface.
+long long fr_hip_shape_op(int op, int dtype, const void *a, const int *a_shape, int a_ndim, const void *b,
+                          const int *b_shape, const int *params, void *out, long long out_capacity_bytes,
+                          int *out_shape, int *out_ndim) {
+  return guarded([&]() -> long long {
+    using namespace rwkv;
+    const DType dt = dtype == 0 ? DType::kFloat32 : dtype == 1 ? DType::kFloat16 : DType::kInt8;
+    auto upload = [&](const void *src, const int *shape, int nd) {
+      Shape sh(shape, shape + nd);
+      Tensor cpu = Tensor::Empty(sh, dt, Device::kCPU);
+      std::memcpy(cpu.data_ptr(), src, cpu.nbytes());
+      return Copy(cpu, Device::kHIP, true);
+    };
+    Tensor x = upload(a, a_shape, a_ndim), y;
+    if (op == 0) {
+      std::vector<Range> r;
+      for (int i = 0; i < a_ndim; i++) r.emplace_back(params[3 * i], params[3 * i + 1], params[3 * i + 2]);
+      y = slice(x, r);
+    } else if (op == 1) {
+      y = cat(x, upload(b, b_shape, a_ndim), params[0]);
+    } else if (op == 2) {
+      y = transpose(x, params[0], params[1]);
+    } else if (op == 3) {
+      y = silu(x);
+    } else {
+      throw FRException("unknown shape op");
+    }
+    Tensor h = Copy(y, Device::kCPU, true);
+    if (static_cast<long long>(h.nbytes()) > out_capacity_bytes) throw FRException("result buffer too small");
+    std::memcpy(out, h.data_ptr(), h.nbytes());
+    *out_ndim = static_cast<int>(h.shape().size());
+    for (int i = 0; i < *out_ndim; i++) out_shape[i] = static_cast<int>(h.size(i));
+    return static_cast<long long>(h.numel());
+  });
+}
+
+// Give the allocator's cached large blocks back to the driver; returns the bytes released.
+long long fr_allocator_trim(void) {
+  return guarded([&]() -> long long { return static_cast<long long>(rwkv::hip::allocator_trim()); });
+}
+
+// One raw allocation / release through the device allocator (tests of reuse, alignment and the
+// out-of-memory path); fr_hip_alloc returns null and sets fr_last_error on failure.
+void *fr_hip_alloc(size_t bytes) {
+  void *p = nullptr;
+  guarded([&]() {
+    p = rwkv::allocator(rwkv::Device::kHIP).Allocate(bytes);
+    return 0;
+  });
+  return p;
+}
+
+int fr_hip_free(void *p) {
+  return guarded([&]() {
+    rwkv::allocator(rwkv::Device::kHIP).Deallocate(p);
     return 0;
   });
 }

@@ -39,11 +39,16 @@ public:
     return p;
   }
 
+  // Called from tensor destructors: must not throw.  A pointer this allocator did not hand out is
+  // reported and dropped.
   void Deallocate(void *ptr) override {
     if (!ptr) return;
     std::lock_guard<std::mutex> lock(_mu);
     auto it = _live.find(ptr);
-    RV_CHECK(it != _live.end()) << "hip allocator: freeing an unknown pointer";
+    if (it == _live.end()) {
+      std::fprintf(stderr, "hip allocator: ignoring the release of an unknown pointer %p\n", ptr);
+      return;
+    }
     const size_t sz = it->second;
     _live.erase(it);
     _in_use -= sz;
@@ -56,14 +61,7 @@ public:
   // Give cached large blocks back to the driver; returns bytes released.
   size_t Trim() {
     std::lock_guard<std::mutex> lock(_mu);
-    size_t freed = 0;
-    for (auto &kv : _large) {
-      frhip_free(kv.second);
-      freed += kv.first;
-    }
-    _large.clear();
-    _reserved -= freed;
-    return freed;
+    return release_large_cache();
   }
 
   size_t reserved() const { return _reserved; }
@@ -75,6 +73,17 @@ private:
     int c = 9;  // 512 B
     while ((size_t(1) << c) < size) c++;
     return c;
+  }
+
+  size_t release_large_cache() {  // caller holds the mutex
+    size_t freed = 0;
+    for (auto &kv : _large) {
+      frhip_free(kv.second);
+      freed += kv.first;
+    }
+    _large.clear();
+    _reserved -= freed;
+    return freed;
   }
 
   void *raw(size_t bytes) {
@@ -91,6 +100,7 @@ private:
     auto &fl = _small[c];
     if (fl.empty()) {
       char *slab = static_cast<char *>(raw(kSlab));
+      if (!slab && release_large_cache() > 0) slab = static_cast<char *>(raw(kSlab));  // last resort, as alloc_large
       if (!slab) return nullptr;
       for (size_t off = 0; off + csz <= kSlab; off += csz) fl.push_back(slab + off);
     }
@@ -113,14 +123,7 @@ private:
       _large.erase(it);
     } else {
       p = raw(rounded);
-      if (!p) {  // last resort: release the cache and retry once
-        for (auto &kv : _large) {
-          frhip_free(kv.second);
-          _reserved -= kv.first;
-        }
-        _large.clear();
-        p = raw(rounded);
-      }
+      if (!p && release_large_cache() > 0) p = raw(rounded);  // last resort: release the cache and retry once
     }
     if (!p) return nullptr;
     _live[p] = got;

@@ -29,6 +29,7 @@ bool device_argmax(Model *model, const Tensor &logits, int *id);
 }  // namespace hip
 namespace def {
 Tensor ModelForward(Model *model, Device device, int id);
+Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids, bool full_output);
 Tensor ModelForwardSeqFallback(Model *model, Device device, const std::vector<int> &ids, bool full_output);
 }  // namespace def
 }  // namespace rwkv

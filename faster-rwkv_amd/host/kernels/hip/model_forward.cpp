@@ -11,7 +11,7 @@
 // (Model::states()) is kept as views of these buffers; states assigned from outside
 // (ResetStates, LoadStateFile, set_states) are copied in on the next call.
 //
-// FR_HIP_GENERIC=1 selects the operator-by-operator loop instead; FR_HIP_NO_GRAPH=1 keeps
+// FR_HIP_GENERIC=1 selects the operator-by-operator loops (one token and seq mode) instead; FR_HIP_NO_GRAPH=1 keeps
 // the fused path but launches eagerly.
 #include <cstdlib>
 #include <cmath>
@@ -41,10 +41,17 @@ struct DecodePlan {
   std::vector<Tensor> aa, bb, pp;       // RWKV-4
   std::vector<Tensor> wkv;              // RWKV-5
   std::vector<Tensor> sx_att[2], sx_ffn[2];
-  std::vector<std::vector<Tensor>> views[2];  // views[parity][layer] = the state tensors model code sees
+  // the state tensors model code sees for shift-state side `side`: (layer, index) -> the plan's buffer
+  Tensor &view(int side, int l, size_t j) {
+    if (j == 0) return sx_att[side][l];
+    if (v5) return j == 1 ? wkv[l] : sx_ffn[side][l];
+    return j == 1 ? aa[l] : j == 2 ? bb[l] : j == 3 ? pp[l] : sx_ffn[side][l];
+  }
+  size_t n_state() const { return v5 ? 3 : 5; }
   int parity = 0;                             // which ping-pong side holds the current shift states
   frhip_graph graph[2] = {nullptr, nullptr};
   bool use_graph = true;
+  bool owned_logits = false;  // FR_HIP_OWNED_LOGITS: Run() returns a tensor of its own instead of a view of the pinned ring
   ~DecodePlan() {
     for (auto g : graph)
       if (g) frhip_graph_destroy(g);
@@ -53,6 +60,26 @@ struct DecodePlan {
       if (h) frhip_host_free(h);
   }
 };
+
+static void alloc_state_buffers(DecodePlan &p) {
+  const int C = p.C;
+  const Device d = Device::kHIP;
+  p.aa.clear(), p.bb.clear(), p.pp.clear(), p.wkv.clear();
+  for (int s = 0; s < 2; s++) p.sx_att[s].clear(), p.sx_ffn[s].clear();
+  for (int l = 0; l < p.L; l++) {
+    if (p.v5) {
+      p.wkv.push_back(Tensor::Empty({p.H, C / p.H, C / p.H}, DType::kFloat32, d));
+    } else {
+      p.aa.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+      p.bb.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+      p.pp.push_back(Tensor::Empty({C}, DType::kFloat32, d));
+    }
+    for (int s = 0; s < 2; s++) {
+      p.sx_att[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
+      p.sx_ffn[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
+    }
+  }
+}
 
 static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   auto p = std::make_shared<DecodePlan>();
@@ -78,30 +105,49 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
     FRHIP_CHECK(frhip_host_malloc(&h, sizeof(float) * (static_cast<size_t>(p->n_logits) + 2 * DecodePlan::kArgmaxBlocks)));
     lh = static_cast<float *>(h);
   }
-  for (int l = 0; l < p->L; l++) {
-    if (p->v5) {
-      p->wkv.push_back(Tensor::Empty({p->H, C / p->H, C / p->H}, DType::kFloat32, d));
-    } else {
-      p->aa.push_back(Tensor::Empty({C}, DType::kFloat32, d));
-      p->bb.push_back(Tensor::Empty({C}, DType::kFloat32, d));
-      p->pp.push_back(Tensor::Empty({C}, DType::kFloat32, d));
-    }
-    for (int s = 0; s < 2; s++) {
-      p->sx_att[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
-      p->sx_ffn[s].push_back(Tensor::Empty({C}, DType::kFloat16, d));
-    }
-  }
-  for (int s = 0; s < 2; s++) {
-    p->views[s].resize(p->L);
-    for (int l = 0; l < p->L; l++) {
-      if (p->v5)
-        p->views[s][l] = {p->sx_att[s][l], p->wkv[l], p->sx_ffn[s][l]};
-      else
-        p->views[s][l] = {p->sx_att[s][l], p->aa[l], p->bb[l], p->pp[l], p->sx_ffn[s][l]};
-    }
-  }
+  alloc_state_buffers(*p);
   p->use_graph = std::getenv("FR_HIP_NO_GRAPH") == nullptr;  // fixed when the model first runs
+  p->owned_logits = std::getenv("FR_HIP_OWNED_LOGITS") != nullptr;
   return p;
+}
+
+// The fused path updates the recurrent state in place, in buffers the plan owns, and Model::states()
+// hands out those buffers.  The reference's operators return fresh tensors every step
+// (kernels/cuda/att.cu:344-353), so a caller may keep a copy of states() as a snapshot and give it back
+// to set_states() later.  To keep that working, a buffer that someone outside still holds (a copy of the
+// States vector shares its storage) is never written again: the plan moves to fresh buffers that start
+// with the current contents, and the captured graphs, which name the old addresses, are dropped.
+static void detach_if_snapshotted(Model *model, DecodePlan &p) {
+  auto &st = model->states();
+  bool held = false;
+  for (int l = 0; l < p.L && !held; l++)
+    for (int side = 0; side < 2 && !held; side++)
+      for (size_t j = 0; j < p.n_state(); j++) {
+        if (side == 1 && j != 0 && j != p.n_state() - 1) continue;  // aa, bb, pp / wkv exist once
+        Tensor &b = p.view(side, l, j);
+        const long expected = 1 + (st[l][j].shares_storage_with(b) ? 1 : 0);
+        if (b.storage_use_count() > expected) {
+          held = true;
+          break;
+        }
+      }
+  if (!held) return;
+  DecodePlan old;  // keeps the old buffers alive until their contents are copied
+  old.v5 = p.v5;
+  old.aa = p.aa, old.bb = p.bb, old.pp = p.pp, old.wkv = p.wkv;
+  for (int s = 0; s < 2; s++) old.sx_att[s] = p.sx_att[s], old.sx_ffn[s] = p.sx_ffn[s];
+  alloc_state_buffers(p);
+  for (int l = 0; l < p.L; l++)
+    for (size_t j = 0; j < p.n_state(); j++) {
+      Tensor &src = old.view(p.parity, l, j), &dst = p.view(p.parity, l, j);
+      FRHIP_CHECK(frhip_memcpy_async(dst.data_ptr(), src.data_ptr(), src.nbytes(), FRHIP_D2D, stream()));
+      if (st[l][j].shares_storage_with(src)) st[l][j] = dst;
+    }
+  FRHIP_CHECK(frhip_stream_sync(stream()));
+  for (auto &g : p.graph) {
+    if (g) frhip_graph_destroy(g);
+    g = nullptr;
+  }
 }
 
 // Bring states assigned from outside into the plan's buffers and rebind the model's
@@ -110,16 +156,16 @@ static void adopt_states(Model *model, DecodePlan &p) {
   auto &st = model->states();
   RV_CHECK(static_cast<int>(st.size()) == p.L);
   for (int l = 0; l < p.L; l++) {
-    auto &mine = p.views[p.parity][l];
-    RV_CHECK(st[l].size() == mine.size());
-    for (size_t j = 0; j < mine.size(); j++) {
-      if (st[l][j].data_ptr() == mine[j].data_ptr()) continue;
-      RV_CHECK(st[l][j].nbytes() == mine[j].nbytes() && st[l][j].dtype() == mine[j].dtype())
+    RV_CHECK(st[l].size() == p.n_state());
+    for (size_t j = 0; j < p.n_state(); j++) {
+      Tensor &mine = p.view(p.parity, l, j);
+      if (st[l][j].data_ptr() == mine.data_ptr()) continue;
+      RV_CHECK(st[l][j].nbytes() == mine.nbytes() && st[l][j].dtype() == mine.dtype())
           << "state " << l << "/" << j << " has the wrong shape or dtype";
       Tensor src = st[l][j].device() == Device::kHIP ? st[l][j] : Copy(st[l][j], Device::kHIP);
-      FRHIP_CHECK(frhip_memcpy_async(mine[j].data_ptr(), src.data_ptr(), src.nbytes(), FRHIP_D2D, stream()));
+      FRHIP_CHECK(frhip_memcpy_async(mine.data_ptr(), src.data_ptr(), src.nbytes(), FRHIP_D2D, stream()));
       if (src.data_ptr() != st[l][j].data_ptr()) FRHIP_CHECK(frhip_stream_sync(stream()));  // src dies here
-      st[l][j] = mine[j];
+      st[l][j] = mine;
     }
   }
 }
@@ -209,6 +255,7 @@ Tensor ModelForward(Model *model, Device device, int id) {
   if (!ex->plan) ex->plan = make_plan(model, *ex);
   DecodePlan &p = *ex->plan;
   RV_CHECK(id >= 0 && id < p.V) << "token id " << id << " out of range";
+  detach_if_snapshotted(model, p);
   adopt_states(model, p);
   frhip_stream s = stream();
   // every call ends with a stream synchronisation, so the device has consumed all earlier slots
@@ -236,8 +283,8 @@ Tensor ModelForward(Model *model, Device device, int id) {
   auto &st = model->states();
   const size_t last = p.v5 ? 2 : 4;
   for (int l = 0; l < p.L; l++) {
-    st[l][0] = p.views[p.parity][l][0];
-    st[l][last] = p.views[p.parity][l][last];
+    st[l][0] = p.view(p.parity, l, 0);
+    st[l][last] = p.view(p.parity, l, last);
   }
   // The head kernel has stored the logits into pinned host memory; waiting for the stream
   // is the step's one synchronisation point (the reference's is the blocking cudaMemcpy in
@@ -258,6 +305,12 @@ Tensor ModelForward(Model *model, Device device, int id) {
     }
     ex->last_argmax = idx < p.n_logits ? idx : 0;
     ex->last_argmax_of = p.logits_host[cur];
+  }
+  if (p.owned_logits) {  // a tensor of the caller's own, as the reference returns (model.cpp:179-186)
+    Tensor out = Tensor::Empty({p.n_logits}, DType::kFloat32, Device::kCPU);
+    std::memcpy(out.data_ptr(), p.logits_host[cur], sizeof(float) * static_cast<size_t>(p.n_logits));
+    ex->last_argmax_of = out.data_ptr();
+    return out;
   }
   return Tensor::FromPtr(p.logits_host[cur], {p.n_logits}, DType::kFloat32, Device::kCPU);
 }
@@ -281,6 +334,8 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
   const std::string &ver = model->version();
   if (std::getenv("FR_HIP_SEQ_FALLBACK") || !(ver == "4" || ver == "5" || ver == "5.2"))
     return def::ModelForwardSeqFallback(model, device, ids, full_output);
+  // the reference-shaped operator loop (vgather, seq operators, slice, layernorm, matmul, cast_dtype)
+  if (std::getenv("FR_HIP_GENERIC")) return def::ModelForwardSeq(model, device, ids, full_output);
   RV_CHECK(!ids.empty());
   auto ex = extra_of(model);
   const int T = static_cast<int>(ids.size()), C = model->n_embd();

@@ -90,11 +90,18 @@ Tensor groupnorm(const Tensor &x, int num_groups, const Tensor &weight, const Te
 Tensor matmul(const Tensor &a, const Tensor &b) {
   RV_CHECK(a.device() == b.device());
   RV_CHECK(a.dtype() == DType::kFloat16) << "matmul on hip: activations are fp16";
-  RV_CHECK(a.sizes().size() == 1 && b.sizes().size() == 2) << "matmul on hip: vector x matrix only on this path";
-  RV_CHECK(a.size(0) == b.size(0)) << "matmul: " << shape_str(a.shape()) << " x " << shape_str(b.shape());
+  RV_CHECK((a.sizes().size() == 1 || a.sizes().size() == 2) && b.sizes().size() == 2)
+      << "matmul on hip: [K] x [K, N] or [T, K] x [K, N]";
+  RV_CHECK(a.size(-1) == b.size(0)) << "matmul: " << shape_str(a.shape()) << " x " << shape_str(b.shape());
   frhip_weight tmp_desc;
   Tensor tmp;
   const frhip_weight *w = weight_of(b, tmp_desc, tmp);
+  if (a.sizes().size() == 2) {  // matrix x matrix (matmul.cpp:110-121): the MFMA product
+    const int T = static_cast<int>(a.size(0));
+    Tensor c = Tensor::Empty({a.size(0), b.size(1)}, a.dtype(), Device::kHIP);
+    FRHIP_CHECK(frhip_gemm(a.data_ptr(), w, c.data_ptr(), T, FRHIP_F16, stream()));
+    return c;
+  }
   Tensor c = Tensor::Empty({b.size(1)}, a.dtype(), Device::kHIP);
   FRHIP_CHECK(frhip_gemv(a.data_ptr(), w, c.data_ptr(), FRHIP_F16, stream()));
   return c;
@@ -114,6 +121,91 @@ Tensor vgather(const std::vector<Tensor> &x, const std::vector<int> &idx) {
     FRHIP_CHECK(frhip_memcpy_async(dst + i * row, x[idx[i]].data_ptr(), row, FRHIP_D2D, stream()));
   }
   return out;
+}
+
+// slice (reference: kernels/cuda/slice.cu:38-136).  Range semantics as there: (0,0,0) is the whole
+// dimension, negative start / end count from the end, output extent (end - start) / interval.
+// Leading-dimension ranges of a contiguous tensor (the last row that model_forward_seq.cpp:171
+// takes, all rows but the last of a token shift) are views into the source, no copy and no launch.
+Tensor slice(const Tensor &x, const std::vector<Range> &ranges) {
+  RV_CHECK(x.sizes().size() == ranges.size() && !ranges.empty() && ranges.size() <= 4);
+  const int nd = static_cast<int>(ranges.size());
+  int src[4], start[4], interval[4], dst[4];
+  Shape out_shape;
+  bool inner_whole = true;  // every dimension after the first is taken whole
+  for (int i = 0; i < nd; i++) {
+    const int dim = static_cast<int>(x.size(i));
+    int st = ranges[i].start, iv = ranges[i].interval, en = ranges[i].end;
+    if (st == 0 && iv == 0 && en == 0) {
+      en = dim;
+      iv = 1;
+    }
+    if (st < 0) st += dim;
+    if (en < 0) en += dim;
+    RV_CHECK(iv > 0);
+    RV_CHECK(st >= 0 && st <= en && en <= dim);
+    src[i] = dim;
+    start[i] = st;
+    interval[i] = iv;
+    dst[i] = (en - st) / iv;
+    out_shape.push_back(dst[i]);
+    if (i > 0 && !(st == 0 && iv == 1 && en == dim)) inner_whole = false;
+  }
+  if (inner_whole && interval[0] == 1 && dst[0] > 0) {
+    const size_t row = x.nbytes() / static_cast<size_t>(src[0]);
+    return Tensor::SubView(x, static_cast<size_t>(start[0]) * row, out_shape);
+  }
+  Tensor out = Tensor::Empty(out_shape, x.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_slice(x.data_ptr(), out.data_ptr(), nd, src, start, interval, dst, x.elem_size(), stream()));
+  return out;
+}
+
+// cat (reference: kernels/cuda/cat.cu:57-111).
+Tensor cat(const Tensor &a, const Tensor &b, int dim) {
+  RV_CHECK(a.sizes().size() == b.sizes().size());
+  RV_CHECK(a.dtype() == b.dtype());
+  RV_CHECK(a.device() == b.device());
+  const int nd = static_cast<int>(a.sizes().size());
+  if (dim < 0) dim += nd;
+  RV_CHECK(dim >= 0 && dim < nd);
+  size_t left = 1, right = 1;
+  Shape out_shape;
+  for (int i = 0; i < nd; i++) {
+    if (i != dim) RV_CHECK(a.size(i) == b.size(i));
+    if (i < dim) left *= static_cast<size_t>(a.size(i));
+    if (i > dim) right *= static_cast<size_t>(a.size(i));
+    out_shape.push_back(i == dim ? a.size(i) + b.size(i) : a.size(i));
+  }
+  Tensor out = Tensor::Empty(out_shape, a.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_cat(a.data_ptr(), b.data_ptr(), out.data_ptr(), left, static_cast<size_t>(a.size(dim)),
+                        static_cast<size_t>(b.size(dim)), right, a.elem_size(), stream()));
+  return out;
+}
+
+// transpose (reference: kernels/cuda/transpose.cu:91-103).
+Tensor transpose(const Tensor &x, int dim_a, int dim_b) {
+  const int nd = static_cast<int>(x.sizes().size());
+  RV_CHECK(nd >= 2 && nd <= 4);
+  if (dim_a < 0) dim_a += nd;
+  if (dim_b < 0) dim_b += nd;
+  RV_CHECK(dim_a >= 0 && dim_b >= 0);
+  RV_CHECK(dim_a < nd && dim_b < nd);
+  Shape out_shape = x.shape();
+  std::swap(out_shape[dim_a], out_shape[dim_b]);
+  int shape[4];
+  for (int i = 0; i < nd; i++) shape[i] = static_cast<int>(x.size(i));
+  Tensor out = Tensor::Empty(out_shape, x.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_transpose(x.data_ptr(), out.data_ptr(), nd, shape, dim_a, dim_b, x.elem_size(), stream()));
+  return out;
+}
+
+// silu (reference: kernels/cuda/activations/silu.cu:38-57; the arithmetic is InplaceSiLU's,
+// kernels/cuda/att.cu:145-152 -- the standalone reference kernel is not SiLU).
+Tensor silu(const Tensor &x) {
+  RV_CHECK(x.dtype() == DType::kFloat16 || x.dtype() == DType::kFloat32);
+  Tensor y = Tensor::Empty(x.shape(), x.dtype(), Device::kHIP);
+  FRHIP_CHECK(frhip_silu(x.data_ptr(), y.data_ptr(), to_frhip_dtype(x.dtype()), static_cast<size_t>(x.numel()), stream()));
+  return y;
 }
 
 // att, RWKV-4 one token (reference: kernels/cuda/att.cu:337-359).
@@ -320,6 +412,10 @@ KernelRegister layernorm_reg("layernorm", Device::kHIP, layernorm);
 KernelRegister groupnorm_reg("groupnorm", Device::kHIP, groupnorm);
 KernelRegister matmul_reg("matmul", Device::kHIP, matmul);
 KernelRegister vgather_reg("vgather", Device::kHIP, vgather);
+KernelRegister slice_reg("slice", Device::kHIP, slice);
+KernelRegister cat_reg("cat", Device::kHIP, cat);
+KernelRegister transpose_reg("transpose", Device::kHIP, transpose);
+KernelRegister silu_reg("silu", Device::kHIP, silu);
 KernelRegister att_reg("att", Device::kHIP, att);
 KernelRegister ffn_reg("ffn", Device::kHIP, ffn);
 KernelRegister ffn_seq_reg("ffn_seq", Device::kHIP, ffn_seq);

@@ -119,6 +119,9 @@ TensorStorage::TensorStorage(size_t nbytes, Device device) : _nbytes(nbytes), _i
 TensorStorage::TensorStorage(void *external_ptr, Device device)
     : _data(external_ptr), _nbytes(0), _is_view(true), _device(device) {}
 
+TensorStorage::TensorStorage(void *ptr_inside, std::shared_ptr<TensorStorage> owner)
+    : _data(ptr_inside), _nbytes(0), _is_view(true), _device(owner->device()), _owner(std::move(owner)) {}
+
 TensorStorage::~TensorStorage() {
   if (!_is_view && _data) allocator(_device).Deallocate(_data);
 }
@@ -151,6 +154,18 @@ Tensor Tensor::FromPtr(void *ptr, const Shape &shape, DType dtype, Device device
 Tensor Tensor::FromOther(const Tensor &other, const Shape &shape) {
   Tensor t;
   t._storage = other._storage;
+  t._shape = shape;
+  t._dtype = other._dtype;
+  t.name = next_name();
+  return t;
+}
+
+Tensor Tensor::SubView(const Tensor &other, size_t byte_offset, const Shape &shape) {
+  RV_CHECK(other.defined());
+  RV_CHECK(byte_offset + static_cast<size_t>(num_elements(shape)) * other.elem_size() <= other.nbytes())
+      << "SubView: range runs past the source tensor";
+  Tensor t;
+  t._storage = std::make_shared<TensorStorage>(static_cast<char *>(other._storage->data_ptr()) + byte_offset, other._storage);
   t._shape = shape;
   t._dtype = other._dtype;
   t.name = next_name();

@@ -70,6 +70,8 @@ class TensorStorage {
 public:
   TensorStorage(size_t nbytes, Device device);       // owns memory from allocator(device)
   TensorStorage(void *external_ptr, Device device);  // view: never frees
+  // view into another storage, which it keeps alive
+  TensorStorage(void *ptr_inside, std::shared_ptr<TensorStorage> owner);
   ~TensorStorage();
   void *data_ptr() const { return _data; }
   Device device() const { return _device; }
@@ -81,6 +83,7 @@ private:
   size_t _nbytes = 0;
   bool _is_view = false;
   Device _device;
+  std::shared_ptr<TensorStorage> _owner;
 };
 
 class Tensor {
@@ -95,6 +98,9 @@ public:
     return static_cast<T *>(_storage->data_ptr());
   }
   bool defined() const { return static_cast<bool>(_storage); }
+  // Number of tensors (and sub-views) that share this tensor's storage, this one included.
+  long storage_use_count() const { return _storage.use_count(); }
+  bool shares_storage_with(const Tensor &other) const { return _storage && _storage == other._storage; }
   DType dtype() const { return _dtype; }
   Device device() const { return _storage->device(); }
   const Shape &sizes() const { return _shape; }
@@ -117,6 +123,8 @@ public:
   static Tensor Empty(const Shape &shape, DType dtype, Device device);
   static Tensor FromPtr(void *ptr, const Shape &shape, DType dtype, Device device);
   static Tensor FromOther(const Tensor &other, const Shape &shape);
+  // A tensor of `shape` (other's dtype) starting `byte_offset` bytes into `other`; shares its storage.
+  static Tensor SubView(const Tensor &other, size_t byte_offset, const Shape &shape);
 
   std::string name;
   bool is_constant = false;

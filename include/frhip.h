@@ -116,6 +116,23 @@ int frhip_scalar_div_f16(void *x, float divisor, size_t n, frhip_stream s);
 /* vgather of embedding rows: kernels/default/gather_ops.cpp:46-89.  table [V][C]; ids on the device. */
 int frhip_gather_rows(const void *table, const int32_t *ids_dev, void *out, int n_ids, int row_bytes, frhip_stream s);
 
+/* slice: kernels/cuda/slice.cu:38-136.  dst[i] = src[start + i * interval] per dimension, ndim 1..4;
+ * the caller has resolved negative / whole-dimension ranges (slice.cu:54-66) into start, interval and
+ * dst_shape.  Shapes travel as kernel arguments: no device allocation or blocking copy per call (the
+ * reference makes four of each, slice.cu:79-111).  elem_bytes 1, 2 or 4. */
+int frhip_slice(const void *src, void *dst, int ndim, const int *src_shape, const int *start, const int *interval,
+                const int *dst_shape, int elem_bytes, frhip_stream s);
+/* cat along one dimension: kernels/cuda/cat.cu:57-111.  a is [left][a_mid][right], b [left][b_mid][right]. */
+int frhip_cat(const void *a, const void *b, void *out, size_t left, size_t a_mid, size_t b_mid, size_t right,
+              int elem_bytes, frhip_stream s);
+/* transpose of two dimensions: kernels/cuda/transpose.cu:36-103.  shape [ndim], ndim 1..4. */
+int frhip_transpose(const void *src, void *dst, int ndim, const int *shape, int dim_a, int dim_b, int elem_bytes,
+                    frhip_stream s);
+/* silu: kernels/cuda/activations/silu.cu:38-57 in name and signature; the arithmetic is that of the
+ * reference's fused path, x / (1 + half(exp(-x))) in half (kernels/cuda/att.cu:145-152) -- the
+ * standalone reference kernel evaluates x / (1 - exp(x)) (silu.cu:19,28), which is not SiLU. */
+int frhip_silu(const void *x, void *y, int dtype, size_t n, frhip_stream s);
+
 /* Token feed for a replayed graph: reads ring[*counter % ring_len] (ring may be pinned host
  * memory, written by the host before the launch), advances *counter on the device, and copies
  * that row of `table` to `out`.  Ids outside [0, n_rows) are clamped.  Replaces the per-token
@@ -247,7 +264,8 @@ int frhip_att_seq_v5(int T, int C, int H, const void *x, const void *sx, const f
                      const frhip_weight *ow,
                      void *x_out, void *xx_out, float *s_out, void *workspace, frhip_stream s_);
 
-/* ---- bandwidth probes (measurement aids, no counterpart in the reference) --------- */
+/* ---- bandwidth probes: DIAGNOSTICS, not operators (measurement aids of bench.py and of the
+ *      hardware-counter calibration; no counterpart in the reference, nothing on the model path calls them) */
 /* Plain device copy, 16 bytes per lane: the kernel of known traffic (bytes read + bytes
  * written) against which hardware counters are scaled. */
 int frhip_copy_probe(void *dst, const void *src, size_t bytes, frhip_stream s);
