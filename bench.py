@@ -42,6 +42,13 @@ CONFIGS = {
 }
 L_, C_, F_, V_ = 24, 2048, 8192, 65536
 
+# HBM bytes per token (fetched + written) by hardware counters, and the profile that records the runs
+TRAFFIC = {
+    "fp16": (2915.2e6 + 2.3e6, "profiles/decode_rwkv4_1b5_fp16_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; "
+                                "not re-read in this run)"),
+    "int8": (None, None),
+}
+
 
 def algorithmic_bytes_per_token(wbytes):
     """Bytes the matrix-vector kernels must move per token: every matrix weight once, plus
@@ -247,6 +254,48 @@ def cpu_baseline(seconds_budget=20.0):
                       "%d+%d tokens timed; per-layer time x24 + head" % (n2, n1)}
 
 
+def probe_mfma(fr, iters=20000, reps=3):
+    """What the matrix cores of this GPU sustain on nothing but v_mfma_f32_32x32x16_f16 (register operands,
+    no memory traffic), with all-zero and with random operands: TFLOP/s from HIP events and the core clock
+    each wave saw (core-clock ticks / 100 MHz ticks of its loop)."""
+    import numpy as np
+    lib = fr.lib()
+    fr.init()
+    name = C.create_string_buffer(128)
+    cus = C.c_int()
+    fr.check(lib.frhip_device_info(name, 128, C.byref(cus), None))
+    st = C.c_void_p()
+    fr.check(lib.frhip_stream_create(C.byref(st)))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.frhip_event_create(C.byref(e0))
+    lib.frhip_event_create(C.byref(e1))
+    rng = np.random.default_rng(0)
+    out = {"compute_units": cus.value, "mfma_per_wave": iters * 6}
+    for waves in (4, 8):
+        sink = fr.DevBuf(cus.value * waves * 64 * 4)
+        clocks = fr.DevBuf.empty((cus.value * waves, 2), np.uint64)
+        for label, data in (("zero", np.zeros((4096, 2, 8), np.float16)),
+                            ("random", rng.standard_normal((4096, 2, 8)).astype(np.float16))):
+            ops = fr.DevBuf.from_numpy(data)
+            fr.check(lib.frhip_mfma_probe(waves, iters, ops.ptr, sink.ptr, clocks.ptr, st))
+            fr.check(lib.frhip_stream_sync(st))
+            best = 1e9
+            for _ in range(reps):
+                fr.check(lib.frhip_event_record(e0, st))
+                fr.check(lib.frhip_mfma_probe(waves, iters, ops.ptr, sink.ptr, clocks.ptr, st))
+                fr.check(lib.frhip_event_record(e1, st))
+                fr.check(lib.frhip_event_sync(e1))
+                ms = C.c_float()
+                fr.check(lib.frhip_event_elapsed_ms(e0, e1, C.byref(ms)))
+                best = min(best, ms.value)
+            ck = clocks.numpy().astype(np.float64)
+            flop = cus.value * waves * iters * 6 * 32768.0
+            out["%dwaves_%s" % (waves, label)] = {"ms": round(best, 3), "TFLOPs": round(flop / (best * 1e-3) / 1e12, 1),
+                                                  "core_clock_MHz": round(float(np.median(ck[:, 0] / ck[:, 1])) * 100.0, 0)}
+    lib.frhip_stream_destroy(st)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -256,6 +305,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the int8-decode and prefill side measurements")
     ap.add_argument("--probe", action="store_true", help="only run the read/copy bandwidth probes and print them")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="only run the matrix-core rate probe (zero vs random operands) and print it")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run the T=1024 seq-mode prefill side measurement and print it (profiling aid)")
     args = ap.parse_args()
@@ -268,6 +319,9 @@ def main():
     fr = importlib.import_module("faster-rwkv_amd")
     if args.probe:
         print(json.dumps(probe_bandwidth(fr)), flush=True)
+        return
+    if args.mfma_probe:
+        print(json.dumps(probe_mfma(fr)), flush=True)
         return
     if args.prefill_only:
         print(json.dumps(prefill_extra(fr)), flush=True)
@@ -290,9 +344,11 @@ def main():
     abytes = algorithmic_bytes_per_token(cfg["wbytes"])
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
     # HBM bytes per launch (average over the launches of one token) from the FETCH_SIZE / WRITE_SIZE
-    # hardware counters, scaled by a copy kernel of known size: measured with rocprofv3 --pmc on this
-    # command and kept in profiles/decode_rwkv4_1b5_fp16_hbm_traffic.md; not measured for uint8.
-    traffic = round((2915.2e6 + 2.3e6) / n_launch) if args.dtype == "fp16" else None
+    # hardware counters, scaled by a copy kernel of known size.  Counters cannot be read inside this
+    # run: the figures are those of the rocprofv3 --pmc runs of this command recorded in the named
+    # profile (they change only when the kernels' access pattern does) and are labelled as such.
+    traffic_bytes_per_token, traffic_source = TRAFFIC[args.dtype]
+    traffic = round(traffic_bytes_per_token / n_launch) if traffic_bytes_per_token else None
     out = {
         "metric": "decode tok/s (RWKV-4 1.5B-shaped, bs1, greedy)", "value": round(tok_s, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -302,7 +358,7 @@ def main():
         "config": {"workload": cfg["workload"], "strategy": cfg["strategy"], "steps": args.steps,
                    "host_loop": "Model::Run (the head stores logits and 64 per-slice arg-max pairs to pinned host memory) + host reduction of the pairs per token"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "row-streaming matrix-vector kernels (att_front/att_out/ffn_front/ffn_out/head), "
                                "%d launches per token" % n_launch,
                      "bytes_per_token": abytes, "kernel_ms_per_token": round(kernel_ms, 4),
@@ -322,6 +378,24 @@ def main():
         extra[other + "_decode_tok_s"] = round(args.steps / osecs, 2)
         extra[other + "_gemv_GBs"] = round(ob / (okms * 1e-3) / 1e9, 1)
         extra[other + "_gemv_frac_of_hbm_peak"] = round(ob / (okms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        # companions of the headline: the same loop over 512 steps when the run was shorter, and with
+        # Model::Run returning a tensor of its own (FR_HIP_OWNED_LOGITS=1) instead of a view of pinned memory
+        if args.dtype == "fp16":
+            if args.steps < 512:
+                lm = fr.Model(cfg["spec"], cfg["strategy"])
+                lm.greedy(0, 16)
+                _, lsecs = lm.greedy(17, 512)
+                lm.close()
+                extra["fp16_decode_tok_s_512_steps"] = round(512 / lsecs, 2)
+            os.environ["FR_HIP_OWNED_LOGITS"] = "1"
+            try:
+                wm = fr.Model(cfg["spec"], cfg["strategy"])
+                wm.greedy(0, 16)
+                _, wsecs = wm.greedy(17, 512)
+                wm.close()
+            finally:
+                del os.environ["FR_HIP_OWNED_LOGITS"]
+            extra["fp16_decode_tok_s_owned_logits"] = round(512 / wsecs, 2)
         extra.update(prefill_extra(fr))
         extra.update(rwkv5_extra(fr))
         extra.update(probe_bandwidth(fr))

@@ -100,6 +100,7 @@ _SIGS = {
     "frhip_gemm_act": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
     "frhip_copy_probe": (_i, [_vp, _vp, _sz, _vp]),
     "frhip_read_probe": (_i, [_vp, _sz, _vp, _vp]),
+    "frhip_mfma_probe": (_i, [_i, _i, _vp, _vp, _vp, _vp]),
     "frhip_seq_workspace_bytes": (_sz, [_i, _i, _i]),
     "frhip_ffn_seq": (_i, [_i, _i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),
     "frhip_att_seq_v4": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),

@@ -342,6 +342,39 @@ int dequant_u8_group_async(int nseg, const unsigned char* const* q, const h1* co
   return check_launch("dequant_u8 (group)");
 }
 
+// ---- matrix-core rate probe (diagnostic) -----------------------------------------------------
+// Nothing but v_mfma_f32_32x32x16_f16 on register operands: six independent accumulators per wave
+// so that the matrix pipe never waits for a result.  Each wave also reads the core clock counter
+// and the constant 100 MHz counter around its loop, which gives the clock the compute unit ran at.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(512) void mfma_probe_kernel(const h8* __restrict__ operands, int iters, float* __restrict__ sink,
+                                                         unsigned long long* __restrict__ clocks) {
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  const h8 a = operands[2 * (gid & 4095)], b = operands[2 * (gid & 4095) + 1];
+  f32x16 acc[6];
+#pragma unroll
+  for (int i = 0; i < 6; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) acc[i][j] = 0.f;
+  const unsigned long long c0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 6; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+  }
+  const unsigned long long c1 = clock64(), w1 = wall_clock64();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < 6; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) t += acc[i][j];
+  sink[gid] = t;
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    const int w = gid / kWave;
+    clocks[2 * w] = c1 - c0;
+    clocks[2 * w + 1] = w1 - w0;
+  }
+}
+
 // ---- shape operators (kernels/cuda/slice.cu:17-36, cat.cu:28-52, transpose.cu:16-34) ----------
 // Index math over at most four dimensions with the shapes passed by value: no device allocation
 // and no blocking copy per call.
@@ -655,6 +688,14 @@ int frhip_silu(const void* x, void* y, int dtype, size_t n, frhip_stream s) {
   else
     return set_error(FRHIP_EINVAL, "silu: dtype must be F16 or F32");
   return check_launch("silu");
+}
+
+int frhip_mfma_probe(int waves_per_workgroup, int iters, const void* operands, void* sink, void* clocks, frhip_stream s) {
+  if (!operands || !sink || !clocks) return set_error(FRHIP_EINVAL, "mfma_probe: null pointer");
+  if (waves_per_workgroup < 1 || waves_per_workgroup > 8 || iters < 1) return set_error(FRHIP_EINVAL, "mfma_probe: 1..8 waves, iters >= 1");
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(compute_units()), dim3(waves_per_workgroup * kWave), 0, static_cast<hipStream_t>(s),
+                     (const h8*)operands, iters, (float*)sink, (unsigned long long*)clocks);
+  return check_launch("mfma_probe");
 }
 
 }  // extern "C"

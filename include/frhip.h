@@ -274,6 +274,13 @@ int frhip_copy_probe(void *dst, const void *src, size_t bytes, frhip_stream s);
  * (at least 8192 bytes): the read-only ceiling the row-streaming kernels are compared with. */
 int frhip_read_probe(const void *src, size_t bytes, void *sink, frhip_stream s);
 
+/* Matrix-core rate probe: one workgroup of `waves_per_workgroup` (1..8) wavefronts per compute unit, each
+ * issuing iters x 6 independent v_mfma_f32_32x32x16_f16 on register operands taken from `operands`
+ * (4096 x 2 x 16 bytes of binary16: all zero, or random, which is what decides the clock the part
+ * sustains).  sink: one float per thread; clocks: per wave {core-clock ticks, 100 MHz ticks} of the loop.
+ * FLOP per launch = compute units x waves x iters x 6 x 32768. */
+int frhip_mfma_probe(int waves_per_workgroup, int iters, const void *operands, void *sink, void *clocks, frhip_stream s);
+
 /* greedy sampler step (Sampler::Sample with top_k = 1, chat.cpp:76-77): index of the
  * largest logit, first one on ties, written to *out_id on the device. */
 int frhip_argmax_f32(const float *logits, int n, int32_t *out_id, frhip_stream s);
