@@ -279,13 +279,49 @@ __global__ __launch_bounds__(64) void wkv4_carry_kernel(Wkv4Seq a) {
   }
 }
 
+// CARRY: the chunk forms its own start state by composing, in order, the incoming state with the
+// local end states of the chunks before it -- the serial pass's arithmetic, step for step, so the
+// results are the serial pass's bit for bit -- instead of reading what wkv4_carry_kernel left.  Chunk j
+// spends j compositions (two exponentials each) where the serial pass spends one launch and nchunk
+// dependent steps per channel; the local states are requested eight chunks at a time.
+template <bool CARRY>
 __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
-  const int c = blockIdx.x * 256 + threadIdx.x, ch = blockIdx.y;
+  // the chunks with the longest prefix first: they decide when the launch ends
+  const int c = blockIdx.x * 256 + threadIdx.x, ch = CARRY ? (int)(gridDim.y - 1 - blockIdx.y) : (int)blockIdx.y;
   if (c >= a.C) return;
   const int t0 = ch * a.Lc, t1 = min(t0 + a.Lc, a.T);
   const float w = a.w[c], u = a.u[c];
   const size_t o = (size_t)ch * a.C + c;
-  float aa = a.sa[o], bb = a.sb[o], pp = a.sp[o];
+  float aa, bb, pp;
+  if constexpr (CARRY) {
+    constexpr int PF = 8;
+    aa = a.aa[c], bb = a.bb[c], pp = a.pp[c];
+    const float pdw = (float)a.Lc * w;  // every chunk before this one is a full chunk
+    for (int j0 = 0; j0 < ch; j0 += PF) {
+      float lp[PF], la[PF], lb[PF];
+#pragma unroll
+      for (int i = 0; i < PF; i++) {
+        const int j = j0 + i < ch ? j0 + i : ch - 1;
+        const size_t q = (size_t)j * a.C + c;
+        lp[i] = a.lp[q];
+        la[i] = a.la[q];
+        lb[i] = a.lb[q];
+      }
+#pragma unroll
+      for (int i = 0; i < PF; i++) {
+        if (j0 + i < ch) {
+          const float pd = pp + pdw;
+          const float p = (pd > lp[i]) ? pd : lp[i];
+          const float e1 = expf(pd - p), e2 = expf(lp[i] - p);
+          aa = e1 * aa + e2 * la[i];
+          bb = e1 * bb + e2 * lb[i];
+          pp = p;
+        }
+      }
+    }
+  } else {
+    aa = a.sa[o], bb = a.sb[o], pp = a.sp[o];
+  }
   for (int tb = t0; tb < t1; tb += kScanB) {
     float kk[kScanB], vv[kScanB];
     h1 rr[kScanB];
@@ -640,6 +676,11 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   Wkv4Seq q;
   q.T = T; q.C = C;
   q.Lc = pick_chunk(T, (C + 255) / 256);
+  // FRHIP_WKV4_SERIAL_CARRY=1: the chunk start states from a serial pass of their own (same bits)
+  static const bool serial_carry = getenv("FRHIP_WKV4_SERIAL_CARRY") != nullptr;
+  // a chunk composes the local states of all chunks before it: half as many, twice as long chunks
+  // (32 of 32 steps at T = 1024) cost the scans less than they save the composition
+  if (!serial_carry && q.Lc < 32 && T >= 512) q.Lc = 32;
   q.nchunk = (T + q.Lc - 1) / q.Lc;
   q.k = w.f0; q.v = w.f1; q.u = t_first; q.w = t_decay; q.r = w.m3;
   q.aa = aa; q.bb = bb; q.pp = pp;
@@ -648,8 +689,12 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   q.aa_out = aa_out; q.bb_out = bb_out; q.pp_out = pp_out;
   dim3 grid((C + 255) / 256, q.nchunk);
   hipLaunchKernelGGL(wkv4_local_kernel, grid, dim3(256), 0, st, q);
-  hipLaunchKernelGGL(wkv4_carry_kernel, dim3((C + 63) / 64), dim3(64), 0, st, q);
-  hipLaunchKernelGGL(wkv4_apply_kernel, grid, dim3(256), 0, st, q);
+  if (serial_carry) {
+    hipLaunchKernelGGL(wkv4_carry_kernel, dim3((C + 63) / 64), dim3(64), 0, st, q);
+    hipLaunchKernelGGL(wkv4_apply_kernel<false>, grid, dim3(256), 0, st, q);
+  } else {
+    hipLaunchKernelGGL(wkv4_apply_kernel<true>, grid, dim3(256), 0, st, q);
+  }
   FR_TRY(check_launch("wkv4_seq"));
 
   GemmArgs b;
