@@ -46,7 +46,8 @@ L_, C_, F_, V_ = 24, 2048, 8192, 65536
 TRAFFIC = {
     "fp16": (2915.2e6 + 2.3e6, "profiles/decode_rwkv4_1b5_fp16_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; "
                                 "not re-read in this run)"),
-    "int8": (None, None),
+    "int8": (1503.8e6 + 2.3e6, "profiles/decode_rwkv4_1b5_int8_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; "
+                                "not re-read in this run)"),
 }
 
 

@@ -16,12 +16,18 @@ struct Model {
   Model(const std::string &path, const std::string &strategy);
   Model(const std::string &path, const std::string &strategy, std::any extra);
   // One id -> one-token forward; several -> seq mode.  Logits come back on the CPU (fp32).
+  // On the hip device the one-token result is a view of one of two pinned host buffers: it stays
+  // valid until the next-but-one Run().  Copy it to keep it longer, or set FR_HIP_OWNED_LOGITS=1
+  // to get a tensor that owns its memory from every call.
   Tensor Run(const std::vector<int> &ids);
   Tensor Run(int id);
   void LoadStateFile(const std::string &path);
   void SaveStateFile(const std::string &path);
   void ResetStates();
   void set_states(const States &states) { _states = states; }
+  // On the hip device these are tensors over the buffers the next forward writes in place.  A copy
+  // of the returned States held by the caller is a snapshot: the next forward moves the model to
+  // fresh buffers first, so set_states(copy) later restores the values at the time of the copy.
   const States &states() const { return _states; }
   States &states() { return _states; }
   // Holds the number of heads, as upstream (kernels/default/init_model.cpp:67).
