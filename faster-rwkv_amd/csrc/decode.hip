@@ -38,6 +38,8 @@ namespace frhip {
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kMaxSeg = 4;
+constexpr int kFusedMaxC = 8 * kThreads;  // widest vector the fused layernorm prologues take
+constexpr int kMaxC = 16384;
 
 struct WMat {
   const unsigned char* data;
@@ -113,6 +115,18 @@ struct Split {
   int base, rem;
 };
 
+// Index of this wave among the waves of the grid, for dealing out work with split_even.  Where the
+// items do not divide evenly the first `rem` indices get one more: numbering the waves across the
+// workgroups first (wave 0 of every workgroup, then wave 1 of every workgroup, ...) spreads those
+// over all compute units instead of loading the first ones with eight longer waves each and leaving
+// the last ones short (ffn_front of the 1.5B shape, 1708 batches for 2048 waves: 10.2 -> 9.4 us).
+// An even split keeps neighbouring rows in neighbouring waves of one workgroup (att_out: 3.6 us
+// against 3.8 us numbered the other way).
+__device__ __forceinline__ int grid_wave(Split sp) {
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  return sp.rem != 0 ? wv * (int)gridDim.x + (int)blockIdx.x : (int)blockIdx.x * kWaves + wv;
+}
+
 __device__ __forceinline__ void split_even(Split sp, int i, int& lo, int& hi) {
   lo = i * sp.base + (i < sp.rem ? i : sp.rem);
   hi = lo + sp.base + (i < sp.rem ? 1 : 0);
@@ -155,6 +169,26 @@ struct RowBatch {
     }
   }
 
+  // The same for a slice of rows longer than one register tiling: chunk j of the slice lies `sbase`
+  // bytes + (j * 64 + lane) chunks into the row.  The slice's byte offset goes into the scalar offset
+  // of the load, and the extents passed in end where the slice ends, so chunks of the tiling that the
+  // slice does not use read zeros without a memory access, like any other tail.
+  __device__ __forceinline__ void load_slice(const void* const (&rows)[R], const int (&nbytes)[R], int lane, int sbase) {
+    __amdgpu_buffer_rsrc_t rs[R];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+      rs[r] = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(rows[r]), 0, nbytes[r], 0x00020000);
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs[r], lane * 16 + (j & 3) * (kWave * 16),
+                                                              sbase + (j >> 2) * (4 * kWave * 16), 2 /* nontemporal */);
+        w[r][j] = __builtin_bit_cast(V, v);
+      }
+    }
+  }
+
   // Chunks of a batch requested ahead of the prologue.  A compute unit keeps only so many bytes of
   // loads in flight (about 64 KB: 8 per wave); a wave that asks for more is held at the load
   // instruction until earlier data has returned, and the older four waves of a workgroup go first.
@@ -175,9 +209,15 @@ struct RowBatch {
   __device__ __forceinline__ void dot_shared(const void* xv, int lane, float (&acc)[R]) const {
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
+    dot_add(xv, lane, 0, kPadChunks, acc);
+  }
+
+  // acc[r] += the products of this batch against chunks c0 + lane + j * 64 of a staged vector of
+  // `padchunks` chunks (the stride between the four 16-byte groups of a uint8 chunk).
+  __device__ __forceinline__ void dot_add(const void* xv, int lane, int c0, int padchunks, float (&acc)[R]) const {
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-      const int c = lane + j * kWave;
+      const int c = c0 + lane + j * kWave;
       if constexpr (!U8) {
         const h8 x = reinterpret_cast<const h8*>(xv)[c];
 #pragma unroll
@@ -189,7 +229,7 @@ struct RowBatch {
         for (int r = 0; r < R; r++) e[r] = o[r] = 0.f;
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
-          const f32x4 x = xp[jj * kPadChunks];
+          const f32x4 x = xp[jj * padchunks];
 #pragma unroll
           for (int r = 0; r < R; r++) {
             const uint32_t word = w[r][j][jj];
@@ -321,7 +361,7 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
 
   const int lane = threadIdx.x & (kWave - 1);
   // wave-uniform, and known to the compiler as such: row addresses stay in scalar registers
-  const int gw = blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int gw = grid_wave(a.split);
   int c0, c1;
   split_even(a.split, gw, c0, c1);
   const size_t row_bytes = U8 ? (size_t)C : 2 * (size_t)C;
@@ -607,7 +647,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // The wave index is made visibly uniform: otherwise the lookups in the kernel arguments
   // (segment table, row addresses) become vector loads that every weight load has to wait for.
   int g0, g1;
-  split_even(a.split, blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), g0, g1);
+  split_even(a.split, grid_wave(a.split), g0, g1);
 
   struct Meta {
     int seg, loc0, nvalid;  // segment, first row within it, rows of the batch that exist
@@ -758,6 +798,44 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
             stage_q(reinterpret_cast<float*>(vec_at(0)), g, kPad, cx[p], cry[p], cmy[p], part);
         }
       }
+    } else if (PRO == P_LN && K > kFusedMaxC) {
+      // a vector wider than one group per thread (the head of a model with n_embd > 4096): the same
+      // normalisation with every thread looping over its groups; x is re-read from the cache
+      const h8* xp8 = reinterpret_cast<const h8*>(a.x);
+      float s1 = 0.f;
+      for (int g = threadIdx.x; g < ngrp; g += kThreads) {
+        const h8 x = xp8[g];
+#pragma unroll
+        for (int i = 0; i < 8; i++) s1 += (float)x[i];
+      }
+      const float mean = block_sum1<kWaves>(s1, red) / (float)K;
+      float s2 = 0.f;
+      for (int g = threadIdx.x; g < ngrp; g += kThreads) {
+        const h8 x = xp8[g];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const float d = (float)x[i] - mean;
+          s2 += d * d;
+        }
+      }
+      float var = block_sum1<kWaves>(s2, red + kWaves) / (float)K;
+      var = var > 0.f ? var : 0.f;
+      const float inv = 1.0f / sqrtf(var + 1e-5f);
+      for (int g = threadIdx.x; g < ngrp; g += kThreads) {
+        const h8 x = xp8[g], gm = reinterpret_cast<const h8*>(a.ln_w)[g], bt = reinterpret_cast<const h8*>(a.ln_b)[g];
+        h8 xx;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const h1 n = (h1)(((float)x[i] - mean) * inv);
+          xx[i] = (n * gm[i]) + bt[i];
+        }
+        if constexpr (!U8) {
+          reinterpret_cast<h8*>(vec_at(0))[g] = xx;
+        } else {
+          const h8 ry = reinterpret_cast<const h8*>(a.seg[0].w.ry)[g], my = reinterpret_cast<const h8*>(a.seg[0].w.my)[g];
+          stage_q(reinterpret_cast<float*>(vec_at(0)), g, kPad, xx, ry, my, part);
+        }
+      }
     } else {
       LnOut ln = ln_regs(xv, lg, lb, own, K, red);
       if (ln.active) {
@@ -823,6 +901,182 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
         g += 1;
       }
     }
+  }
+}
+
+// ===========================================================================
+// WKV-4 update of one token as a kernel of its own (kernels/cuda/att.cu:30-62), one thread per
+// channel: the arithmetic of att_front_v4_kernel's last step, for models wider than that
+// kernel takes.  r has already passed through the sigmoid.
+// ===========================================================================
+struct Wkv4One {
+  int C;
+  const float *k, *v, *aa, *bb, *pp, *td, *tf;
+  const h1* r;
+  h1* rwkv_out;
+  float *aa_out, *bb_out, *pp_out;
+};
+
+__global__ __launch_bounds__(256) void wkv4_one_kernel(Wkv4One a) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= a.C) return;
+  const float k = a.k[n], v = a.v[n];
+  const h1 r = a.r[n];
+  float ww = a.tf[n] + k;
+  const float pp_ = a.pp[n];
+  float p_ = (pp_ > ww) ? pp_ : ww;
+  float e1 = expf(pp_ - p_);
+  float e2 = expf(ww - p_);
+  const float aa_ = a.aa[n], bb_ = a.bb[n];
+  const float wkv = (e1 * aa_ + e2 * v) / (e1 * bb_ + e2);
+  a.rwkv_out[n] = r * (h1)wkv;
+  ww = a.td[n] + pp_;
+  p_ = (ww > k) ? ww : k;
+  e1 = expf(ww - p_);
+  e2 = expf(k - p_);
+  a.aa_out[n] = e1 * aa_ + e2 * v;
+  a.bb_out[n] = e1 * bb_ + e2;
+  a.pp_out[n] = p_;
+}
+
+// ===========================================================================
+// Rows longer than the largest register tiling (K > 9216 binary16 / 16384 uint8 elements: the
+// ffn value matrix of the 3B and larger models).  One matrix against one ready vector (P_COPY).
+// A workgroup owns consecutive rows; a row is cut into `nslice` slices of `cs` chunks per lane
+// (cs <= NCH), and the (row, slice) items of the workgroup are dealt evenly to its eight waves,
+// so that the waves stay balanced also where the matrix has fewer rows than the grid has waves.
+// A wave streams its items through two alternating register sets and leaves one partial sum
+// per item in LDS; after a barrier one thread per row adds the row's partials in slice order
+// (a fixed order: results do not depend on timing) and runs the epilogue.
+// The whole vector is staged in LDS (2 K bytes; uint8: 4 K bytes of x * ry in fp32).
+// ===========================================================================
+struct SliceGeom {
+  int nslice, cs;    // slices per row, chunks per lane and slice
+  int padchunks;     // chunks of the staged vector, padding included: (nslice - 1) * cs * 64 + NCH * 64
+  Split rows;        // rows over the workgroups of the grid
+  int part_offset;   // byte offset of the partial sums in dynamic LDS
+};
+
+template <int NCH, bool U8>
+__global__ __launch_bounds__(kThreads) void rows_sliced_kernel(RowsArgs a, SliceGeom g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ float qred[kWaves][kMaxSeg * kQSums];
+  const int K = a.K;
+  const int nchunk = U8 ? (K >> 4) : (K >> 3);
+  const int row_bytes = U8 ? K : 2 * K;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const Seg& sg = a.seg[0];
+  const int N = sg.w.N;
+  float* partials = reinterpret_cast<float*>(smem + g.part_offset);
+  int r0, r1;  // this workgroup's rows
+  split_even(g.rows, blockIdx.x, r0, r1);
+  const int nrows = r1 - r0;
+  const int items = nrows * g.nslice;
+  const int i0 = (int)(((long)items * wv) / kWaves), i1 = (int)(((long)items * (wv + 1)) / kWaves);
+
+  // per-row operands of the epilogue, thread t holding those of row r0 + t (first pass of the final loop)
+  h1 ex = (h1)0.0f, er = (h1)0.0f, qrx = (h1)0.0f, qmx = (h1)0.0f;
+  if ((int)threadIdx.x < nrows) {
+    const int n = r0 + threadIdx.x;
+    const int ri = n < a.res_n ? n : a.res_n - 1;
+    ex = a.res_x[ri];
+    er = a.res_r[ri];
+    if constexpr (U8) {
+      qrx = sg.w.rx[n];
+      qmx = sg.w.mx[n];
+    }
+  }
+
+  // item -> (row, slice); the slice's extent ends where the slice does
+  auto fetch = [&](RowBatch<1, NCH, U8>& b, int row, int sl, bool live) {
+    const void* rows[1] = {sg.w.data + (size_t)(live ? row : 0) * (size_t)row_bytes};
+    const int end = (sl + 1) * g.cs * (kWave * 16);
+    const int nbytes[1] = {live ? (end < row_bytes ? end : row_bytes) : 0};
+    b.load_slice(rows, nbytes, lane, sl * g.cs * (kWave * 16));
+  };
+
+  RowBatch<1, NCH, U8> A, B;
+  int row = r0 + i0 / g.nslice, sl = i0 % g.nslice;
+  fetch(A, row, sl, i0 < i1);
+
+  // ---- the vector, staged under the first loads ----
+  float part[kQSums] = {0.f, 0.f};
+  for (int gi = threadIdx.x; gi < (K >> 3); gi += kThreads) {
+    const h8 x = reinterpret_cast<const h8*>(a.vec0)[gi];
+    if constexpr (!U8) {
+      reinterpret_cast<h8*>(smem)[gi] = x;
+    } else {
+      const h8 ry = reinterpret_cast<const h8*>(sg.w.ry)[gi];
+      const h8 my = reinterpret_cast<const h8*>(sg.w.my)[gi];
+      stage_q(reinterpret_cast<float*>(smem), gi, g.padchunks, x, ry, my, part);
+    }
+  }
+  zero_pad<U8>(smem, nchunk, g.padchunks);
+  if constexpr (U8) publish_qsums(part, kQSums, qred);
+  __syncthreads();
+  float qtv = 0.f;
+  if constexpr (U8) qtv = gather_qsums(kQSums, qred);
+
+  auto consume = [&](const RowBatch<1, NCH, U8>& b, int row_, int sl_) {
+    float acc[1] = {0.f};
+    b.dot_add(smem, lane, sl_ * g.cs * kWave, g.padchunks, acc);
+    const float t = wave_sum(acc[0]);
+    if (lane == 0) partials[(row_ - r0) * g.nslice + sl_] = t;
+  };
+  auto advance = [&](int& r_, int& s_) {
+    s_ += 1;
+    if (s_ == g.nslice) {
+      s_ = 0;
+      r_ += 1;
+    }
+  };
+  // fetch the next item, consume the current one; the two register sets alternate
+  for (int i = i0; i < i1;) {
+    int nrow = row, nsl = sl;
+    advance(nrow, nsl);
+    if (i + 1 >= i1) {
+      consume(A, row, sl);
+      break;
+    }
+    fetch(B, nrow, nsl, true);
+    consume(A, row, sl);
+    row = nrow;
+    sl = nsl;
+    i += 1;
+    advance(nrow, nsl);
+    if (i + 1 >= i1) {
+      consume(B, row, sl);
+      break;
+    }
+    fetch(A, nrow, nsl, true);
+    consume(B, row, sl);
+    row = nrow;
+    sl = nsl;
+    i += 1;
+  }
+  __syncthreads();
+
+  // ---- one thread per row: partials in slice order, then the epilogue ----
+  for (int t = threadIdx.x; t < nrows; t += kThreads) {
+    const int n = r0 + t;
+    if (t >= kThreads) {  // more rows than threads: operands of the later passes
+      const int ri = n < a.res_n ? n : a.res_n - 1;
+      ex = a.res_x[ri];
+      er = a.res_r[ri];
+      if constexpr (U8) {
+        qrx = sg.w.rx[n];
+        qmx = sg.w.mx[n];
+      }
+    }
+    float sum = 0.f;
+    for (int s_ = 0; s_ < g.nslice; s_++) sum += partials[t * g.nslice + s_];
+    if constexpr (U8) {
+      const float q0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), 0));
+      const float q1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), 1));
+      sum = finish_q(sum, (float)qrx, (float)qmx, q0, q1);
+    }
+    run_epilogue(a, sg, n, sum, ex, er);
   }
 }
 
@@ -923,9 +1177,12 @@ static int check_vec(const void* p, const char* what) {
     if (_e != 0) return _e; \
   } while (0)
 
+// The fused one-token kernels hold the activation vector as one 8-element group per thread; wider
+// models run the same arithmetic as separate launches (layernorm + mixes, one product per matrix,
+// state update), which costs them a few launches per layer where a launch moves 50 MB and more.
 static int check_embd(int C) {
-  if (C <= 0 || C % 16 != 0 || C > 8 * kThreads)
-    return set_error(FRHIP_ESHAPE, "n_embd must be a multiple of 16 and at most 4096");
+  if (C <= 0 || C % 16 != 0 || C > kMaxC)
+    return set_error(FRHIP_ESHAPE, "n_embd must be a multiple of 16 and at most 16384");
   return 0;
 }
 
@@ -1043,9 +1300,87 @@ static Split make_split(int total, int grid) {
   return Split{total / waves, total % waves};
 }
 
+// Rows too long for a register tiling: slices of at most kSliceNch chunks per lane.
+constexpr int kSliceNch = 8;
+constexpr size_t kSlicedMaxLds = 144 * 1024;
+
+// Dynamic LDS above 64 KB has to be allowed per kernel and device; frhip_init does it for the
+// device it initialises, outside any stream capture.
+int allow_large_lds() {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rows_sliced_kernel<kSliceNch, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSlicedMaxLds);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rows_sliced_kernel<kSliceNch, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSlicedMaxLds);
+  if (e != hipSuccess) return set_error((int)e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+  return 0;
+}
+
+// Chunks per lane and slice: the choice that wastes least, counting both the chunks of the last
+// slice that lie beyond the row and the waves that get one item fewer than the others.
+static size_t sliced_lds(int cs, int nslice, int rows_per_wg, bool u8) {
+  const size_t padchunks = (size_t)(nslice - 1) * cs * kWave + kSliceNch * kWave;
+  return padchunks * (u8 ? 64 : 16) + (size_t)rows_per_wg * nslice * sizeof(float);
+}
+
+// (among the choices whose staged vector and partial sums fit the LDS; none: *cs_out stays 0)
+static void pick_slices(int total_chunks, int rows_per_wg, bool u8, int* cs_out, int* nslice_out) {
+  double best = -1.0;
+  *cs_out = 0;
+  for (int cs = kSliceNch; cs >= 4; cs--) {
+    const int nslice = (total_chunks + cs - 1) / cs;
+    if (sliced_lds(cs, nslice, rows_per_wg, u8) > kSlicedMaxLds) continue;
+    const long items = (long)rows_per_wg * nslice;
+    const long per_wave = (items + kWaves - 1) / kWaves;
+    const double eff = ((double)total_chunks / ((double)nslice * cs)) * ((double)items / (double)(per_wave * kWaves));
+    if (eff > best + 1e-9) {
+      best = eff;
+      *cs_out = cs;
+      *nslice_out = nslice;
+    }
+  }
+}
+
+static int launch_rows_sliced(const RowsArgs& args, bool u8, hipStream_t st, const char* what) {
+  if (args.prologue != P_COPY || args.nseg != 1)
+    return set_error(FRHIP_ESHAPE, "row-streaming kernel: K above 9216 (binary16) / 16384 (uint8) is supported for one matrix "
+                                   "against a ready vector only");
+  RowsArgs a = args;
+  if (!a.res_x || !a.res_r) {
+    const h1* any = reinterpret_cast<const h1*>(a.seg[0].w.data);
+    if (!a.res_x && !a.res_r) a.res_n = 1;
+    if (!a.res_x) a.res_x = a.res_r ? a.res_r : any;
+    if (!a.res_r) a.res_r = a.res_x;
+  }
+  const int grid = decode_grid();
+  const int N = a.seg[0].w.N;
+  const int rows_per_wg = (N + grid - 1) / grid;
+  SliceGeom g;
+  pick_slices(chunks_per_lane(a.K, u8), rows_per_wg, u8, &g.cs, &g.nslice);
+  if (g.cs == 0)
+    return set_error(FRHIP_ESHAPE, "row-streaming kernel: K or N is too large for the long-row kernel's LDS (144 KB)");
+  g.padchunks = (g.nslice - 1) * g.cs * kWave + kSliceNch * kWave;
+  g.rows = Split{N / grid, N % grid};
+  const size_t vec_bytes = (size_t)g.padchunks * (u8 ? 64 : 16);
+  g.part_offset = (int)vec_bytes;
+  const size_t lds = vec_bytes + (size_t)rows_per_wg * g.nslice * sizeof(float);
+  if (lds > kSlicedMaxLds)
+    return set_error(FRHIP_ESHAPE, "row-streaming kernel: K or N is too large for the long-row kernel's LDS (144 KB)");
+  if (u8)
+    hipLaunchKernelGGL((rows_sliced_kernel<kSliceNch, true>), dim3(grid), dim3(kThreads), lds, st, a, g);
+  else
+    hipLaunchKernelGGL((rows_sliced_kernel<kSliceNch, false>), dim3(grid), dim3(kThreads), lds, st, a, g);
+  return check_launch(what);
+}
+
 static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char* what) {
   const int nch = round_nch(chunks_per_lane(args.K, u8));
-  if (nch < 0) return set_error(FRHIP_ESHAPE, "K is too large for the row-streaming kernel (max 9216 fp16 / 18432 uint8)");
+  // the staged vector of a uint8 product takes 4 K bytes of LDS: where that and the kernel's static LDS pass 64 KB the
+  // sliced kernel (which may use more) takes over
+  if (nch < 0 || staged_bytes(nch, u8) + 1024 > 64 * 1024) return launch_rows_sliced(args, u8, st, what);
+  static const int sliced_from = env_int("FRHIP_SLICED_FROM_K", 0);  // measurement switch: long-row kernel from this K on
+  if (sliced_from > 0 && args.K >= sliced_from && args.prologue == P_COPY && args.nseg == 1)
+    return launch_rows_sliced(args, u8, st, what);
   const int grid = decode_grid();
   RowsArgs a = args;
   // epilogue operands are read unconditionally: point unused ones at any readable element
@@ -1101,22 +1436,36 @@ static void add_seg(RowsArgs& a, const frhip_weight* w, int vec, int epi, void* 
   a.nseg = s + 1;
 }
 
+// One matrix against a ready vector, with an epilogue: the building block of the operators of
+// models wider than the fused kernels take.
+static int product(const frhip_weight* w, const h1* vec, int epi, void* out, hipStream_t st, const char* what) {
+  RowsArgs a = empty_args(w->K);
+  a.prologue = P_COPY;
+  a.nvec = 1;
+  a.vec0 = vec;
+  add_seg(a, w, 0, epi, out);
+  return launch_rows(a, w->dtype == FRHIP_U8, st, what);
+}
+
 }  // namespace frhip
 
 using namespace frhip;
 
 extern "C" size_t frhip_decode_workspace_bytes(int C, int F) {
-  // binary16 rwkv [C] | r [C] | x_mid [C] | g [C] ; fp32 k [C] | v [C] | r32 [C] ; binary16 vx [F];
-  // each 256-byte aligned (g, k, v, r32 serve RWKV-5 only)
+  // binary16 rwkv [C] | r [C] | x_mid [C] | g [C] ; fp32 k [C] | v [C] | r32 [C] ; (n_embd > 4096: four
+  // mixed vectors, binary16 [C] each) ; binary16 vx [F]; each 256-byte aligned
   auto al = [](size_t n) { return (n + 255) / 256 * 256; };
   if (C <= 0 || F <= 0) return 0;
-  return al(2 * (size_t)C) * 4 + al(2 * (size_t)F) + al(4 * (size_t)C) * 3;
+  // models wider than the fused kernels take (n_embd > 4096) also keep their four mixed vectors here
+  const size_t wide = C > kFusedMaxC ? al(2 * (size_t)C) * 4 : 0;
+  return al(2 * (size_t)C) * 4 + al(2 * (size_t)F) + al(4 * (size_t)C) * 3 + wide;
 }
 
 namespace {
 struct Workspace {
   h1 *rwkv, *r, *vx, *xmid, *g;
   float *k32, *v32, *r32;
+  h1* mixed[4];  // n_embd > 4096 only
 };
 Workspace carve(void* ws, int C) {
   auto al = [](size_t n) { return (n + 255) / 256 * 256; };
@@ -1136,7 +1485,11 @@ Workspace carve(void* ws, int C) {
   p += al(4 * (size_t)C);
   w.r32 = reinterpret_cast<float*>(p);
   p += al(4 * (size_t)C);
-  w.vx = reinterpret_cast<h1*>(p);
+  for (int i = 0; i < 4; i++) {
+    w.mixed[i] = reinterpret_cast<h1*>(p);
+    if (C > kFusedMaxC) p += al(2 * (size_t)C);
+  }
+  w.vx = reinterpret_cast<h1*>(p);  // [F], the only part whose size the attention operators do not know: last
   return w;
 }
 }  // namespace
@@ -1204,6 +1557,30 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   Workspace w = carve(workspace, C);
   const int grid = decode_grid();
 
+  if (C > kFusedMaxC) {
+    const void* mixes[3] = {k_mix, v_mix, r_mix};
+    void* outs[3] = {w.mixed[0], w.mixed[1], w.mixed[2]};
+    FR_TRY(launch_ln_mix(1, C, x, sx, ln_w, ln_b, mixes, outs, 3, xx_out, st));
+    FR_TRY(product(kw, w.mixed[0], E_STORE_F32, w.k32, st, "att_k"));
+    FR_TRY(product(vw, w.mixed[1], E_STORE_F32, w.v32, st, "att_v"));
+    FR_TRY(product(rw, w.mixed[2], E_SIGMOID, w.r, st, "att_r"));
+    Wkv4One q;
+    q.C = C;
+    q.k = w.k32; q.v = w.v32; q.aa = aa; q.bb = bb; q.pp = pp; q.td = t_decay; q.tf = t_first;
+    q.r = w.r; q.rwkv_out = w.rwkv;
+    q.aa_out = aa_out; q.bb_out = bb_out; q.pp_out = pp_out;
+    hipLaunchKernelGGL(wkv4_one_kernel, dim3((C + 255) / 256), dim3(256), 0, st, q);
+    FR_TRY(check_launch("wkv4_one"));
+    RowsArgs b = empty_args(C);
+    b.prologue = P_COPY;
+    b.nvec = 1;
+    b.vec0 = w.rwkv;
+    b.res_x = (const h1*)x;
+    b.res_n = C;
+    add_seg(b, ow, 0, E_RESIDUAL, x_out);
+    return launch_rows(b, ow->dtype == FRHIP_U8, st, "att_out");
+  }
+
   AttFrontV4 a;
   a.C = C;
   a.split = make_split(C, grid);
@@ -1218,17 +1595,25 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   const int nch_t = nch <= 1 ? 1 : nch == 2 ? 2 : nch <= 4 ? 4 : nch == 5 ? 5 : 8;  // compiled tilings
   const size_t lds = staged_bytes(nch_t, u8) * 3;
   FR_TRY(check_lds(lds));
-  const bool single = C <= grid * kWaves;
-#define FR_ATT_FRONT(N)                                                                                   \
-  do {                                                                                                    \
-    if (u8 && single)                                                                                     \
-      hipLaunchKernelGGL((att_front_v4_kernel<N, true, true>), dim3(grid), dim3(kThreads), lds, st, a);   \
-    else if (u8)                                                                                          \
-      hipLaunchKernelGGL((att_front_v4_kernel<N, true, false>), dim3(grid), dim3(kThreads), lds, st, a);  \
-    else if (single)                                                                                      \
-      hipLaunchKernelGGL((att_front_v4_kernel<N, false, true>), dim3(grid), dim3(kThreads), lds, st, a);  \
-    else                                                                                                  \
-      hipLaunchKernelGGL((att_front_v4_kernel<N, false, false>), dim3(grid), dim3(kThreads), lds, st, a); \
+  // More channels than one workgroup per CU has waves (n_embd 2560 ... 4096): one channel per wave over
+  // up to two workgroups per CU instead of a loop over two channels in some waves -- the loop's second set
+  // of rows does not fit the registers beside the first for long rows, so its loads would wait for the
+  // first channel's products.
+  static const bool two_wgs = env_int("FRHIP_ATT_TWO_WGS", 1) == 1;
+  int grid_a = grid;
+  if (two_wgs && C > grid * kWaves && C <= 2 * grid * kWaves) grid_a = (C + kWaves - 1) / kWaves;
+  const bool single = C <= grid_a * kWaves;
+  a.split = make_split(C, grid_a);
+#define FR_ATT_FRONT(N)                                                                                     \
+  do {                                                                                                      \
+    if (u8 && single)                                                                                       \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, true, true>), dim3(grid_a), dim3(kThreads), lds, st, a);   \
+    else if (u8)                                                                                            \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, true, false>), dim3(grid_a), dim3(kThreads), lds, st, a);  \
+    else if (single)                                                                                        \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, false, true>), dim3(grid_a), dim3(kThreads), lds, st, a);  \
+    else                                                                                                    \
+      hipLaunchKernelGGL((att_front_v4_kernel<N, false, false>), dim3(grid_a), dim3(kThreads), lds, st, a); \
   } while (0)
   if (nch <= 1) FR_ATT_FRONT(1);
   else if (nch == 2) FR_ATT_FRONT(2);
@@ -1281,17 +1666,27 @@ static int att_one_v5_impl(bool v50, int C, int H, const void* x, const void* sx
   Workspace w = carve(workspace, C);
 
   // LN -> 4 mixes -> k, v, r (fp32) and g = silu(.) (half)      att.cu:276-290
-  RowsArgs a = empty_args(C);
-  a.prologue = P_LN_MIX;
-  a.nvec = v50 ? 3 : 4;
-  a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
-  a.mix[0] = (const h1*)k_mix; a.mix[1] = (const h1*)v_mix; a.mix[2] = (const h1*)r_mix; a.mix[3] = (const h1*)g_mix;
-  a.xx_out = (h1*)xx_out;
-  add_seg(a, kw, 0, E_STORE_F32, w.k32);
-  add_seg(a, vw, 1, E_STORE_F32, w.v32);
-  add_seg(a, rw, 2, E_STORE_F32, w.r32);
-  if (!v50) add_seg(a, gw, 3, E_SILU, w.g);
-  FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "att_v5_front"));
+  if (C > kFusedMaxC) {
+    const void* mixes[4] = {k_mix, v_mix, r_mix, g_mix};
+    void* outs[4] = {w.mixed[0], w.mixed[1], w.mixed[2], w.mixed[3]};
+    FR_TRY(launch_ln_mix(1, C, x, sx, ln_w, ln_b, mixes, outs, v50 ? 3 : 4, xx_out, st));
+    FR_TRY(product(kw, w.mixed[0], E_STORE_F32, w.k32, st, "att_v5_k"));
+    FR_TRY(product(vw, w.mixed[1], E_STORE_F32, w.v32, st, "att_v5_v"));
+    FR_TRY(product(rw, w.mixed[2], E_STORE_F32, w.r32, st, "att_v5_r"));
+    if (!v50) FR_TRY(product(gw, w.mixed[3], E_SILU, w.g, st, "att_v5_g"));
+  } else {
+    RowsArgs a = empty_args(C);
+    a.prologue = P_LN_MIX;
+    a.nvec = v50 ? 3 : 4;
+    a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+    a.mix[0] = (const h1*)k_mix; a.mix[1] = (const h1*)v_mix; a.mix[2] = (const h1*)r_mix; a.mix[3] = (const h1*)g_mix;
+    a.xx_out = (h1*)xx_out;
+    add_seg(a, kw, 0, E_STORE_F32, w.k32);
+    add_seg(a, vw, 1, E_STORE_F32, w.v32);
+    add_seg(a, rw, 2, E_STORE_F32, w.r32);
+    if (!v50) add_seg(a, gw, 3, E_SILU, w.g);
+    FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "att_v5_front"));
+  }
 
   Wkv5One k;
   k.H = H;
@@ -1355,16 +1750,24 @@ extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const 
   hipStream_t st = static_cast<hipStream_t>(s);
   Workspace w = carve(workspace, C);
 
-  RowsArgs a = empty_args(C);
-  a.prologue = P_LN_MIX;
-  a.nvec = 2;
-  a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
-  a.mix[0] = (const h1*)r_mix;
-  a.mix[1] = (const h1*)k_mix;
-  a.xx_out = (h1*)xx_out;
-  add_seg(a, rw, 0, E_SIGMOID, w.r);
-  add_seg(a, kw, 1, E_RELU2, w.vx);
-  FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "ffn_front"));
+  if (C > kFusedMaxC) {
+    const void* mixes[2] = {r_mix, k_mix};
+    void* outs[2] = {w.mixed[0], w.mixed[1]};
+    FR_TRY(launch_ln_mix(1, C, x, sx, ln_w, ln_b, mixes, outs, 2, xx_out, st));
+    FR_TRY(product(rw, w.mixed[0], E_SIGMOID, w.r, st, "ffn_r"));
+    FR_TRY(product(kw, w.mixed[1], E_RELU2, w.vx, st, "ffn_k"));
+  } else {
+    RowsArgs a = empty_args(C);
+    a.prologue = P_LN_MIX;
+    a.nvec = 2;
+    a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+    a.mix[0] = (const h1*)r_mix;
+    a.mix[1] = (const h1*)k_mix;
+    a.xx_out = (h1*)xx_out;
+    add_seg(a, rw, 0, E_SIGMOID, w.r);
+    add_seg(a, kw, 1, E_RELU2, w.vx);
+    FR_TRY(launch_rows(a, kw->dtype == FRHIP_U8, st, "ffn_front"));
+  }
 
   RowsArgs b = empty_args(F);
   b.prologue = P_COPY;

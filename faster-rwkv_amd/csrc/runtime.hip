@@ -84,6 +84,7 @@ int frhip_init(int device) {
   }
   g_cus = 0;
   compute_units();
+  if (int e = allow_large_lds()) return e;
   return static_scratch(nullptr);  // this device's copy of the built-in scratch
 }
 

@@ -122,7 +122,9 @@ def test_dequant_random_matrix_bit_exact(K, N):
     assert np.array_equal(out.numpy().T.view(np.uint16), po.dequant_u8(q, mx, rx, my, ry).view(np.uint16))
 
 
-@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 8192), (8192, 2048), (2560, 2560), (8960, 2560), (768, 50277), (64, 3), (16, 1)])
+# K above 9216 (binary16) / 16384 (uint8): rows consumed in slices
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 8192), (8192, 2048), (2560, 2560), (8960, 2560), (768, 50277), (64, 3), (16, 1),
+                                 (10240, 2560), (16384, 515), (20480, 130), (32768, 9), (9232, 33)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_gemv_against_oracle(K, N, quant):
     x = h(rng.standard_normal(K))
