@@ -905,6 +905,69 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
 }
 
 // ===========================================================================
+// Layernorm of one token's vector and its token-shift mixes as a kernel of its own, for models
+// wider than the fused prologues take (n_embd > 4096): out[i] = mix(LN(x), sx, mix[i]) for
+// i < nmix, xx_out = LN(x)   (kernels/cuda/layer_norm.cu:60-69, att.cu:90-113).
+// One workgroup; thread t owns the 8-element groups t, t + 512, ... (at most four: n_embd <= 16384).
+// ===========================================================================
+struct LnMixOne {
+  int C, nmix;
+  const h1 *x, *sx, *ln_w, *ln_b;
+  const h1* mix[4];
+  h1* out[4];
+  h1* xx_out;
+};
+
+__global__ __launch_bounds__(kThreads) void ln_mix_one_kernel(LnMixOne a) {
+  constexpr int G = kMaxC / (8 * kThreads);
+  __shared__ float red[2 * kWaves];
+  const int ngrp = a.C >> 3;
+  h8 xv[G], gm[G], bt[G], sx[G];
+  bool own[G];
+#pragma unroll
+  for (int i = 0; i < G; i++) {
+    const int g = threadIdx.x + i * kThreads;
+    own[i] = g < ngrp;
+    const int gc = own[i] ? g : 0;
+    xv[i] = reinterpret_cast<const h8*>(a.x)[gc];
+    gm[i] = reinterpret_cast<const h8*>(a.ln_w)[gc];
+    bt[i] = reinterpret_cast<const h8*>(a.ln_b)[gc];
+    sx[i] = reinterpret_cast<const h8*>(a.sx)[gc];
+  }
+  float s1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < G; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) s1 += own[i] ? (float)xv[i][e] : 0.f;
+  const float mean = block_sum1<kWaves>(s1, red) / (float)a.C;
+  float s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < G; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float d = (float)xv[i][e] - mean;
+      s2 += own[i] ? d * d : 0.f;
+    }
+  float var = block_sum1<kWaves>(s2, red + kWaves) / (float)a.C;
+  var = var > 0.f ? var : 0.f;
+  const float inv = 1.0f / sqrtf(var + 1e-5f);
+#pragma unroll
+  for (int i = 0; i < G; i++) {
+    if (!own[i]) continue;
+    const int g = threadIdx.x + i * kThreads;
+    h8 xx;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const h1 n = (h1)(((float)xv[i][e] - mean) * inv);
+      xx[e] = (n * gm[i][e]) + bt[i][e];
+    }
+    reinterpret_cast<h8*>(a.xx_out)[g] = xx;
+    for (int m = 0; m < a.nmix; m++)
+      reinterpret_cast<h8*>(a.out[m])[g] = mix8(xx, sx[i], reinterpret_cast<const h8*>(a.mix[m])[g]);
+  }
+}
+
+// ===========================================================================
 // WKV-4 update of one token as a kernel of its own (kernels/cuda/att.cu:30-62), one thread per
 // channel: the arithmetic of att_front_v4_kernel's last step, for models wider than that
 // kernel takes.  r has already passed through the sigmoid.
@@ -1436,6 +1499,21 @@ static void add_seg(RowsArgs& a, const frhip_weight* w, int vec, int epi, void* 
   a.nseg = s + 1;
 }
 
+static int launch_ln_mix_one(int C, const void* x, const void* sx, const void* ln_w, const void* ln_b,
+                             const void* const* mix, h1* const* out, int nmix, void* xx_out, hipStream_t st) {
+  LnMixOne a;
+  a.C = C;
+  a.nmix = nmix;
+  a.x = (const h1*)x; a.sx = (const h1*)sx; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
+  for (int i = 0; i < 4; i++) {
+    a.mix[i] = i < nmix ? (const h1*)mix[i] : nullptr;
+    a.out[i] = i < nmix ? out[i] : nullptr;
+  }
+  a.xx_out = (h1*)xx_out;
+  hipLaunchKernelGGL(ln_mix_one_kernel, dim3(1), dim3(kThreads), 0, st, a);
+  return check_launch("ln_mix_one");
+}
+
 // One matrix against a ready vector, with an epilogue: the building block of the operators of
 // models wider than the fused kernels take.
 static int product(const frhip_weight* w, const h1* vec, int epi, void* out, hipStream_t st, const char* what) {
@@ -1559,8 +1637,7 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
 
   if (C > kFusedMaxC) {
     const void* mixes[3] = {k_mix, v_mix, r_mix};
-    void* outs[3] = {w.mixed[0], w.mixed[1], w.mixed[2]};
-    FR_TRY(launch_ln_mix(1, C, x, sx, ln_w, ln_b, mixes, outs, 3, xx_out, st));
+    FR_TRY(launch_ln_mix_one(C, x, sx, ln_w, ln_b, mixes, w.mixed, 3, xx_out, st));
     FR_TRY(product(kw, w.mixed[0], E_STORE_F32, w.k32, st, "att_k"));
     FR_TRY(product(vw, w.mixed[1], E_STORE_F32, w.v32, st, "att_v"));
     FR_TRY(product(rw, w.mixed[2], E_SIGMOID, w.r, st, "att_r"));
@@ -1595,13 +1672,14 @@ extern "C" int frhip_att_one_v4(int C, const void* x, const void* sx, const floa
   const int nch_t = nch <= 1 ? 1 : nch == 2 ? 2 : nch <= 4 ? 4 : nch == 5 ? 5 : 8;  // compiled tilings
   const size_t lds = staged_bytes(nch_t, u8) * 3;
   FR_TRY(check_lds(lds));
-  // More channels than one workgroup per CU has waves (n_embd 2560 ... 4096): one channel per wave over
-  // up to two workgroups per CU instead of a loop over two channels in some waves -- the loop's second set
-  // of rows does not fit the registers beside the first for long rows, so its loads would wait for the
-  // first channel's products.
+  // uint8 weights, more channels than one workgroup per CU has waves (n_embd 2560 ... 4096): one channel
+  // per wave over up to two workgroups per CU instead of a loop over two channels in some waves.  The loop's
+  // second set of uint8 rows does not fit the registers beside the first, so its loads wait for the first
+  // channel's products (decode of the 3B / 7B widths: 2452 -> 2714, 1704 -> 1906 tok/s over 8 layers; the
+  // binary16 loop, which requests ahead, is as fast or faster than two workgroups: 2696 vs 2625 tok/s).
   static const bool two_wgs = env_int("FRHIP_ATT_TWO_WGS", 1) == 1;
   int grid_a = grid;
-  if (two_wgs && C > grid * kWaves && C <= 2 * grid * kWaves) grid_a = (C + kWaves - 1) / kWaves;
+  if (two_wgs && u8 && C > grid * kWaves && C <= 2 * grid * kWaves) grid_a = (C + kWaves - 1) / kWaves;
   const bool single = C <= grid_a * kWaves;
   a.split = make_split(C, grid_a);
 #define FR_ATT_FRONT(N)                                                                                     \
@@ -1668,8 +1746,7 @@ static int att_one_v5_impl(bool v50, int C, int H, const void* x, const void* sx
   // LN -> 4 mixes -> k, v, r (fp32) and g = silu(.) (half)      att.cu:276-290
   if (C > kFusedMaxC) {
     const void* mixes[4] = {k_mix, v_mix, r_mix, g_mix};
-    void* outs[4] = {w.mixed[0], w.mixed[1], w.mixed[2], w.mixed[3]};
-    FR_TRY(launch_ln_mix(1, C, x, sx, ln_w, ln_b, mixes, outs, v50 ? 3 : 4, xx_out, st));
+    FR_TRY(launch_ln_mix_one(C, x, sx, ln_w, ln_b, mixes, w.mixed, v50 ? 3 : 4, xx_out, st));
     FR_TRY(product(kw, w.mixed[0], E_STORE_F32, w.k32, st, "att_v5_k"));
     FR_TRY(product(vw, w.mixed[1], E_STORE_F32, w.v32, st, "att_v5_v"));
     FR_TRY(product(rw, w.mixed[2], E_STORE_F32, w.r32, st, "att_v5_r"));
@@ -1752,8 +1829,7 @@ extern "C" int frhip_ffn_one(int C, int F, const void* x, const void* sx, const 
 
   if (C > kFusedMaxC) {
     const void* mixes[2] = {r_mix, k_mix};
-    void* outs[2] = {w.mixed[0], w.mixed[1]};
-    FR_TRY(launch_ln_mix(1, C, x, sx, ln_w, ln_b, mixes, outs, 2, xx_out, st));
+    FR_TRY(launch_ln_mix_one(C, x, sx, ln_w, ln_b, mixes, w.mixed, 2, xx_out, st));
     FR_TRY(product(rw, w.mixed[0], E_SIGMOID, w.r, st, "ffn_r"));
     FR_TRY(product(kw, w.mixed[1], E_RELU2, w.vx, st, "ffn_k"));
   } else {

@@ -22,10 +22,5 @@ int compute_units();
 int static_scratch(void** ptr);
 // Lets the long-row kernels of the current device use more than 64 KB of dynamic LDS.
 int allow_large_lds();
-// Rows t = 0 .. T-1 of x ([T][C] binary16) normalised and mixed with the row before them (row -1 is
-// `state`): out[i][t] = mix(LN(x[t]), LN(x[t-1]), mix[i]) for i < nmix, xx_last = LN(x[T-1]).  Any C;
-// with T = 1 it serves the one-token operators of models wider than their fused kernels take.
-int launch_ln_mix(int T, int C, const void* x, const void* state, const void* ln_w, const void* ln_b,
-                  const void* const* mix, void* const* out, int nmix, void* xx_last, hipStream_t st);
 
 }  // namespace frhip

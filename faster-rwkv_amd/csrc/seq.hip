@@ -522,14 +522,14 @@ static int check_w(const frhip_weight* w, int K, int N, const char* what) {
   return 0;
 }
 
-int launch_ln_mix(int T, int C, const void* x, const void* state, const void* ln_w, const void* ln_b,
-                  const void* const* mix, void* const* out, int nmix, void* xx_last, hipStream_t st) {
+static int launch_ln_mix(int T, int C, const void* x, const void* state, const void* ln_w, const void* ln_b,
+                         const void* const* mix, h1* const* out, int nmix, void* xx_last, hipStream_t st) {
   LnMixSeq a;
   a.T = T; a.C = C; a.nmix = nmix;
   a.x = (const h1*)x; a.state = (const h1*)state; a.ln_w = (const h1*)ln_w; a.ln_b = (const h1*)ln_b;
   for (int i = 0; i < nmix; i++) {
     a.mix[i] = (const h1*)mix[i];
-    a.out[i] = static_cast<h1*>(out[i]);
+    a.out[i] = out[i];
   }
   a.xx_last = (h1*)xx_last;
   const int nwg = (T + kLnRows - 1) / kLnRows;
@@ -623,7 +623,7 @@ extern "C" int frhip_ffn_seq(int T, int C, int F, const void* x, const void* sx,
   hipStream_t st = static_cast<hipStream_t>(s);
   SeqWs w = carve_seq(workspace, T, C, F);
   const void* mixes[2] = {k_mix, r_mix};
-  void* outs[2] = {w.m0, w.m1};
+  h1* outs[2] = {w.m0, w.m1};
   FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, 2, xx_out, st));
   GemmArgs a;
   memset(&a, 0, sizeof(a));
@@ -663,7 +663,7 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   hipStream_t st = static_cast<hipStream_t>(s);
   SeqWs w = carve_seq(workspace, T, C, 64);
   const void* mixes[3] = {k_mix, v_mix, r_mix};
-  void* outs[3] = {w.m0, w.m1, w.m2};
+  h1* outs[3] = {w.m0, w.m1, w.m2};
   FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, 3, xx_out, st));
   GemmArgs a;
   memset(&a, 0, sizeof(a));
@@ -728,7 +728,7 @@ static int att_seq_v5_impl(bool v50, int T, int C, int H, const void* x, const v
   hipStream_t st = static_cast<hipStream_t>(s);
   SeqWs w = carve_seq(workspace, T, C, 64);
   const void* mixes[4] = {k_mix, v_mix, r_mix, g_mix};
-  void* outs[4] = {w.m0, w.m1, w.m2, w.m3};
+  h1* outs[4] = {w.m0, w.m1, w.m2, w.m3};
   FR_TRY(launch_ln_mix(T, C, x, sx, ln_w, ln_b, mixes, outs, v50 ? 3 : 4, xx_out, st));
   GemmArgs a;
   memset(&a, 0, sizeof(a));

@@ -148,7 +148,9 @@ def _ffn_one_checks(C_, F_, quant, div2, x, sx, ln_w, ln_b, mk, mr, kw, vw, rw, 
                        zip(out_g.view(np.uint16), r_g.view(np.uint16), x.view(np.uint16))], np.uint16).view(np.float16)
     if div2:
         strict = (strict.astype(np.float32) / 2).astype(np.float16)
-    assert_close_f16(x_out.numpy(), strict, max_ulp=1, max_frac=0.002, what="x_out from kernel intermediates")
+    # (a product of F > 8192 terms is several times the residual it is added to: where the fp32 sum lands on the other
+    # side of a rounding boundary than the exact sum, one spacing of the product is a few spacings of the output)
+    assert_close_f16(x_out.numpy(), strict, max_ulp=1 if F_ <= 8192 else 4, max_frac=0.002, what="x_out from kernel intermediates")
 
 
 @pytest.mark.parametrize("C_,H_", [(2560, 40), (512, 8), (5120, 80)])
