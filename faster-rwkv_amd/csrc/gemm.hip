@@ -370,6 +370,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
 // term moves them one slot apart: SQ_LDS_BANK_CONFLICT is 0 and a read takes 4 cycles (without
 // that term every read was a two-way conflict: 8 cycles).
 // ---------------------------------------------------------------------------
+// global_load_lds_dwordx4 with the address as a scalar base plus a 32-bit lane offset.  The builtin
+// takes a 64-bit address per lane, which costs the loader one vector add per load; on the SIMD it
+// shares with an MFMA wave each of those waits for a gap between that wave's MFMAs, and the whole
+// workgroup waits for the loader at the step's barrier (per K-step of a 128 x 256 tile: loader 2150
+// cycles from barrier to barrier, MFMA waves 1550-1700 plus 540-700 waiting).  In this form a load
+// needs scalar instructions only.  `lds` is the destination's LDS byte address (lane l writes 16 bytes
+// at lds + 16 l); the wait counts are the caller's business, as with the builtin.
+__device__ __forceinline__ void load_lds_saddr(unsigned voff, const void* sbase, unsigned lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory");
+}
+
+// The same address for every lane, in scalar registers (the compiler cannot always prove it).
+__device__ __forceinline__ const unsigned char* uniform_ptr(const void* p) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return reinterpret_cast<const unsigned char*>(((unsigned long long)hi << 32) | lo);
+}
+
 constexpr int kLdwThreads = 320;
 constexpr int kLdwStages = 4;
 constexpr int kLdwBK = 64;
@@ -419,9 +437,26 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
       row = row < N ? row : N - 1;
       pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + kbase + (ls ^ (b & 1)) * 8;
     }
+    // a tile wholly inside the matrices: scalar base per load plus one of two lane offsets (load_lds_saddr)
+    const bool full = m0 + BM <= M && n0 + BN <= N && (size_t)K * 16 + 128 < 0xffffffffull;
+    const unsigned voff[2] = {(unsigned)(lr * K * 2 + ls * 16), (unsigned)(lr * K * 2 + (ls ^ 1) * 16)};
+    const unsigned char* abase = uniform_ptr(reinterpret_cast<const unsigned char*>(sg.A) + ((size_t)m0 * K + kbase) * 2);
+    const unsigned char* bbase = uniform_ptr(reinterpret_cast<const unsigned char*>(sg.B) + ((size_t)n0 * K + kbase) * 2);
+    const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)gemm_smem);
+    const size_t group = (size_t)__builtin_amdgcn_readfirstlane(K) * 16;
     auto issue = [&](int step) {
-      unsigned char* st = gemm_smem + (step % kLdwStages) * kStageBytes;
       const int k0 = step * kLdwBK;
+      if (full) {
+        const unsigned stl = lds0 + (step % kLdwStages) * kStageBytes;
+        const unsigned char* ak = abase + (size_t)k0 * 2;
+        const unsigned char* bk = bbase + (size_t)k0 * 2;
+#pragma unroll
+        for (int b = 0; b < kAInstr; b++) load_lds_saddr(voff[b & 1], ak + b * group, stl + b * 1024);
+#pragma unroll
+        for (int b = 0; b < kBInstr; b++) load_lds_saddr(voff[b & 1], bk + b * group, stl + kABytes + b * 1024);
+        return;
+      }
+      unsigned char* st = gemm_smem + (step % kLdwStages) * kStageBytes;
 #pragma unroll
       for (int b = 0; b < kAInstr; b++)
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pa[b] + k0),
@@ -589,9 +624,27 @@ __device__ __forceinline__ void vw_loader(const GemmSeg& sg, unsigned char* smem
     pb[b] = reinterpret_cast<const h1*>(sg.B) + (size_t)row * K + (ls ^ (b & 1)) * 8;
   }
   const int nk = K / kLdwBK;
+  // a tile that lies wholly inside the matrices: rows are 8 K halves apart for every lane, so the address of
+  // load b is a uniform base (row group b, this step's k) plus one of two lane offsets
+  const bool full = m0 + BM <= M && n0 + W * 32 <= N && (size_t)K * 16 + 128 < 0xffffffffull;
+  const unsigned voff[2] = {(unsigned)(lr * K * 2 + ls * 16), (unsigned)(lr * K * 2 + (ls ^ 1) * 16)};
+  const unsigned char* abase = uniform_ptr(reinterpret_cast<const unsigned char*>(sg.A) + (size_t)m0 * K * 2);
+  const unsigned char* bbase = uniform_ptr(reinterpret_cast<const unsigned char*>(sg.B) + (size_t)n0 * K * 2);
+  const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)smem);
+  const size_t group = (size_t)__builtin_amdgcn_readfirstlane(K) * 16;  // bytes between row groups of 8
   auto issue = [&](int step, int slot) {
-    unsigned char* st = smem + slot * stage_bytes;
     const int k0 = step * kLdwBK;
+    if (full) {
+      const unsigned st = lds0 + slot * stage_bytes;
+      const unsigned char* ak = abase + (size_t)k0 * 2;
+      const unsigned char* bk = bbase + (size_t)k0 * 2;
+#pragma unroll
+      for (int b = 0; b < kAInstr; b++) load_lds_saddr(voff[b & 1], ak + b * group, st + b * 1024);
+#pragma unroll
+      for (int b = 0; b < kBInstr; b++) load_lds_saddr(voff[b & 1], bk + b * group, st + kVwABytes + b * 1024);
+      return;
+    }
+    unsigned char* st = smem + slot * stage_bytes;
 #pragma unroll
     for (int b = 0; b < kAInstr; b++)
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pa[b] + k0),
