@@ -297,6 +297,85 @@ def probe_mfma(fr, iters=20000, reps=3):
     return out
 
 
+_GEMM_SHAPES = ((2048, 6144), (2048, 8192), (2048, 10240), (2048, 2048), (8192, 2048))
+
+_TORCH_YARDSTICK = r"""
+import json, sys, torch
+T, reps = int(sys.argv[1]), int(sys.argv[2])
+out = {}
+for K, N in %s:
+    nrot = max(2, int(600e6 // (K * N * 2)))
+    tw = [torch.randn(N, K, device="cuda", dtype=torch.float16) * 0.02 for _ in range(nrot)]
+    tx = torch.randn(T, K, device="cuda", dtype=torch.float16)
+    for w in tw:
+        tx @ w.t()
+    torch.cuda.synchronize()
+    best = 1e9
+    for _ in range(reps):
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for w in tw:
+            tx @ w.t()
+        t1.record()
+        torch.cuda.synchronize()
+        best = min(best, t0.elapsed_time(t1) * 1e3 / nrot)
+    out["%%dx%%dx%%d" %% (T, K, N)] = round(best, 1)
+    del tw, tx
+print(json.dumps(out))
+""" % (repr(_GEMM_SHAPES),)
+
+
+def probe_gemm(fr, T=1024, reps=4):
+    """The prompt pass's matrix x matrix products one at a time (frhip_gemm, binary16 in and out, no epilogue), on
+    weights that come from HBM (a rotation of matrices larger than the caches), and -- as a yardstick, not as
+    part of the product -- torch.matmul (hipBLASLt / rocBLAS) on the same shapes and operand layout.  torch brings
+    a HIP runtime of its own, so it runs in a child process, before this process touches the GPU."""
+    import subprocess
+    yard = {}
+    try:
+        r = subprocess.run([sys.executable, "-c", _TORCH_YARDSTICK, str(T), str(reps)], capture_output=True, text=True, timeout=300)
+        yard = json.loads(r.stdout.strip().splitlines()[-1]) if r.returncode == 0 else {}
+    except Exception as e:  # no torch, no GPU for it: the yardstick column stays empty
+        print("[bench] torch yardstick not available: %r" % (e,), file=sys.stderr)
+    lib = fr.lib()
+    fr.init()
+    rng = np.random.default_rng(0)
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.frhip_event_create(C.byref(e0))
+    lib.frhip_event_create(C.byref(e1))
+    out = {"T": T, "shapes": {}}
+    for K, N in _GEMM_SHAPES:
+        nrot = max(2, int(600e6 // (K * N * 2)))
+        x = fr.DevBuf.from_numpy(rng.standard_normal((T, K)).astype(np.float16))
+        w_nk = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)  # output-major, as the kernels read weights
+        ws = [fr.DevBuf.from_numpy(w_nk) for _ in range(nrot)]
+        y = fr.DevBuf(T * N * 2)
+        structs = [fr.Weight(w.ptr, None, None, None, None, K, N, fr.F16) for w in ws]
+
+        def run():
+            for wt in structs:
+                fr.check(lib.frhip_gemm(x.ptr, C.byref(wt), y.ptr, T, fr.F16, None))
+        run()
+        fr.check(lib.frhip_device_sync())
+        best = 1e9
+        for _ in range(reps):
+            fr.check(lib.frhip_event_record(e0, None))
+            run()
+            fr.check(lib.frhip_event_record(e1, None))
+            fr.check(lib.frhip_event_sync(e1))
+            ms = C.c_float()
+            fr.check(lib.frhip_event_elapsed_ms(e0, e1, C.byref(ms)))
+            best = min(best, ms.value * 1e3 / nrot)
+        key = "%dx%dx%d" % (T, K, N)
+        row = {"frhip_gemm_us": round(best, 1), "frhip_gemm_TFLOPs": round(2.0 * T * K * N / best * 1e-6, 0)}
+        if key in yard:
+            row["torch_matmul_us"] = yard[key]
+            row["torch_matmul_TFLOPs"] = round(2.0 * T * K * N / yard[key] * 1e-6, 0)
+        out["shapes"][key] = row
+        del ws, structs, x, y
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -308,6 +387,8 @@ def main():
     ap.add_argument("--probe", action="store_true", help="only run the read/copy bandwidth probes and print them")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only run the matrix-core rate probe (zero vs random operands) and print it")
+    ap.add_argument("--gemm-probe", action="store_true",
+                    help="only time the prompt pass's products standalone, beside torch.matmul on the same shapes, and print that")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run the T=1024 seq-mode prefill side measurement and print it (profiling aid)")
     args = ap.parse_args()
@@ -323,6 +404,9 @@ def main():
         return
     if args.mfma_probe:
         print(json.dumps(probe_mfma(fr)), flush=True)
+        return
+    if args.gemm_probe:
+        print(json.dumps(probe_gemm(fr)), flush=True)
         return
     if args.prefill_only:
         print(json.dumps(prefill_extra(fr)), flush=True)
