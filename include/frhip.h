@@ -64,7 +64,8 @@ typedef struct frhip_weight {
 int frhip_abi_version(void);
 const char *frhip_error_string(void);
 int frhip_device_count(int *count);
-int frhip_init(int device);                         /* select device, create handles */
+int frhip_init(int device);                         /* select device, create handles; also lets this device's long-row
+                                                       kernels use more than 64 KB of LDS (K beyond 32768 fp16 elements) */
 int frhip_device_info(char *name, size_t name_len, int *compute_units, size_t *total_mem);
 int frhip_malloc(void **ptr, size_t bytes);         /* hipMalloc; caching sits above, in the host allocator */
 int frhip_free(void *ptr);
@@ -105,7 +106,8 @@ int frhip_dequant_u8(const frhip_weight *w, void *dst_nk_f16, frhip_stream s);
 int frhip_layernorm(const void *x, const void *gamma, const void *beta, void *y, int rows, int cols, int dtype, frhip_stream s);
 /* groupnorm over fp32 rows: kernels/cuda/group_norm.cu:322-357. */
 int frhip_groupnorm_f32(const float *x, int groups, const float *gamma, const float *beta, float *y, int rows, int cols, frhip_stream s);
-/* matmul, vector x matrix: kernels/cuda/matmul.cpp:105-109.  x [K] binary16; y [N] in out_dtype (F16 or F32). */
+/* matmul, vector x matrix: kernels/cuda/matmul.cpp:105-109.  x [K] binary16; y [N] in out_dtype (F16 or F32).
+ * K a multiple of 16, at most 73728 for binary16 and 32768 for uint8 weights. */
 int frhip_gemv(const void *x, const frhip_weight *w, void *y, int out_dtype, frhip_stream s);
 /* cast_dtype: kernels/cuda/cast_dtype.cu:24-41. */
 int frhip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n, frhip_stream s);
@@ -143,7 +145,10 @@ int frhip_embed_ring(const void *table, int n_rows, int row_bytes, const int32_t
 
 /* ---- fused one-token operators ------------------------------------------------ */
 /* Scratch the fused operators need: frhip_decode_workspace_bytes(C, F) bytes,
- * 256-byte aligned, owned by the caller, reusable across calls on one stream. */
+ * 256-byte aligned, owned by the caller, reusable across calls on one stream.
+ * C (n_embd) is a multiple of 16 and at most 16384: up to 4096 an operator is two fused launches,
+ * above that the same arithmetic runs as one launch per matrix (and the workspace holds the mixed
+ * vectors).  F (n_ffn) is a multiple of 16, at most 73728 (binary16) / 32768 (uint8). */
 size_t frhip_decode_workspace_bytes(int C, int F);
 
 /* att (RWKV-4, one token): kernels/cuda/att.cu:182-217,337-359.
