@@ -200,8 +200,12 @@ struct RowBatch {
   // uint8 rows cost two VALU operations per code, about as long as their bytes take to arrive: the
   // sooner the prologue's barrier, the more of the products run under the stream, so only about
   // six loads go first there.
+  // (uint8, re-measured as decode tok/s of the 1.5B RWKV-4 / 8 layers of the 3B RWKV-5.2: about 6 loads first
+  // 1576 / 2808, about 12 first -- the whole batch of the 1.5B shape -- 1515 / 2793, the whole batch of the 3B shape 2686;
+  // binary16: whole batches first 1407 / 2539 against 1445 / 2628 as below, 12 first 1401 / 2628.)
   static constexpr int kFirst = U8 ? 6 : 8;
-  static constexpr int kHead = R * NCH <= (U8 ? 6 : 16) ? NCH : (kFirst / R < 1 ? 1 : kFirst / R);
+  static constexpr int kHead0 = R * NCH <= (U8 ? 6 : 16) ? NCH : (kFirst / R < 1 ? 1 : kFirst / R);
+  static constexpr int kHead = kHead0 < NCH ? kHead0 : NCH;  // never beyond the batch
 
   // All rows against one staged vector, each chunk of which is read from LDS once.  Binary16 rows:
   // acc[r] = sum_k w[k] x[k] against a binary16 vector; uint8 rows: acc[r] = sum_k q[k] xr[k]
