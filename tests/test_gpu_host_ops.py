@@ -17,6 +17,15 @@ from synth import make_model
 fr = importlib.import_module("faster-rwkv_amd")
 rng = np.random.default_rng(2024)
 
+
+@pytest.fixture(autouse=True)
+def _rng_per_test(request):
+    """Every test draws from a generator seeded by its own name, so its data do not depend on which
+    other tests ran before it (or on cases added to them)."""
+    import zlib
+    global rng
+    rng = np.random.default_rng([2024, zlib.crc32(request.node.name.encode())])
+
 SLICE, CAT, TRANSPOSE, SILU = 0, 1, 2, 3
 
 

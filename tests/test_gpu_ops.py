@@ -26,6 +26,15 @@ def keep(a):
 rng = np.random.default_rng(123)
 
 
+@pytest.fixture(autouse=True)
+def _rng_per_test(request):
+    """Every test draws from a generator seeded by its own name, so its data do not depend on which
+    other tests ran before it (or on cases added to them)."""
+    import zlib
+    global rng
+    rng = np.random.default_rng([123, zlib.crc32(request.node.name.encode())])
+
+
 def h(x):
     return np.asarray(x, np.float32).astype(np.float16)
 
@@ -145,9 +154,9 @@ def test_gemv_against_oracle(K, N, quant):
     mag = np.abs(x.astype(np.float64)) @ np.abs(pw.exact())
     assert (np.abs(y32.numpy() - exact) <= 4e-6 * mag + 1e-6).all()
     # ... and within the w^-rounding noise of the oracle, which multiplies by binary16 w^
-    # (relative error up to 2^-12 per element, uniform): six standard deviations of that sum
+    # (relative error up to 2^-12 per element, uniform): eight standard deviations of that sum
     rms = lambda a: float(np.sqrt(np.mean(np.asarray(a, np.float64) ** 2)))
-    noise = 6 * (2.0 ** -12 / np.sqrt(3)) * np.sqrt(K) * rms(x) * rms(wref)
+    noise = 8 * (2.0 ** -12 / np.sqrt(3)) * np.sqrt(K) * rms(x) * rms(wref)
     assert np.abs(y32.numpy() - ref32).max() <= tol + noise + 2e-5
     r16 = ref32.astype(np.float16).astype(np.float32)
     half_spacing = np.exp2(np.floor(np.log2(np.maximum(np.abs(r16), 1e-7))) - 11)

@@ -22,6 +22,15 @@ def keep(a):
 rng = np.random.default_rng(777)
 
 
+@pytest.fixture(autouse=True)
+def _rng_per_test(request):
+    """Every test draws from a generator seeded by its own name, so its data do not depend on which
+    other tests ran before it (or on cases added to them)."""
+    import zlib
+    global rng
+    rng = np.random.default_rng([777, zlib.crc32(request.node.name.encode())])
+
+
 def h(x):
     return np.asarray(x, np.float32).astype(np.float16)
 
