@@ -296,11 +296,13 @@ __device__ __forceinline__ void stage_q(float* dst, int g, int padchunks, h8 x, 
   const int c = g >> 1, j = (g & 1) * 2;
   reinterpret_cast<f32x4*>(dst)[j * nchunk + c] = lo;
   reinterpret_cast<f32x4*>(dst)[(j + 1) * nchunk + c] = hi;
+  // Sx and Smy with the packed dot product (products of two binary16 values are exact in fp32): 8 instructions
+  // instead of 32 conversions, adds and fmas on every workgroup's way to its first product
+  h8 ones;
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    part[0] += (float)x[i];
-    part[1] += (float)x[i] * (float)my[i];
-  }
+  for (int i = 0; i < 8; i++) ones[i] = (h1)1.0f;
+  part[0] = dot8acc(x, ones, part[0]);
+  part[1] = dot8acc(x, my, part[1]);
 }
 
 // Per-wave sums of the nval per-thread partials go to red[wave][v]; the caller's next barrier
