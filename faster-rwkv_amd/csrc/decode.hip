@@ -284,8 +284,8 @@ __device__ __forceinline__ void zero_pad(void* vec, int nchunk, int padchunks) {
 // ---------------------------------------------------------------------------
 constexpr int kQSums = 2;  // Sx, Smy
 
-// Thread-owned group g = 8 consecutive elements of the vector.
-__device__ __forceinline__ void stage_q(float* dst, int g, int padchunks, h8 x, h8 ry, h8 my, float* part) {
+// Thread-owned group g = 8 consecutive elements of the vector: xr = x * ry into the staged vector.
+__device__ __forceinline__ void stage_xr(float* dst, int g, int padchunks, h8 x, h8 ry) {
   const int nchunk = padchunks;
   f32x4 lo, hi;
 #pragma unroll
@@ -296,13 +296,21 @@ __device__ __forceinline__ void stage_q(float* dst, int g, int padchunks, h8 x, 
   const int c = g >> 1, j = (g & 1) * 2;
   reinterpret_cast<f32x4*>(dst)[j * nchunk + c] = lo;
   reinterpret_cast<f32x4*>(dst)[(j + 1) * nchunk + c] = hi;
-  // Sx and Smy with the packed dot product (products of two binary16 values are exact in fp32): 8 instructions
-  // instead of 32 conversions, adds and fmas on every workgroup's way to its first product
+}
+
+// The group's share of Sx = sum x and Smy = sum x my, with the packed dot product (products of two
+// binary16 values are exact in fp32): 8 instructions instead of 32 conversions, adds and fmas.
+__device__ __forceinline__ void sum_q(h8 x, h8 my, float* part) {
   h8 ones;
 #pragma unroll
   for (int i = 0; i < 8; i++) ones[i] = (h1)1.0f;
   part[0] = dot8acc(x, ones, part[0]);
   part[1] = dot8acc(x, my, part[1]);
+}
+
+__device__ __forceinline__ void stage_q(float* dst, int g, int padchunks, h8 x, h8 ry, h8 my, float* part) {
+  stage_xr(dst, g, padchunks, x, ry);
+  sum_q(x, my, part);
 }
 
 // Per-wave sums of the nval per-thread partials go to red[wave][v]; the caller's next barrier
@@ -441,14 +449,15 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   float part[3 * kQSums];
 #pragma unroll
   for (int i = 0; i < 3 * kQSums; i++) part[i] = 0.f;
+  h8 mk{}, mv{}, mr{};
   if (ln.active) {
-    const h8 mk = mix8(ln.xx, sx, mixk);
-    const h8 mv = mix8(ln.xx, sx, mixv);
-    const h8 mr = mix8(ln.xx, sx, mixr);
+    mk = mix8(ln.xx, sx, mixk);
+    mv = mix8(ln.xx, sx, mixv);
+    mr = mix8(ln.xx, sx, mixr);
     if constexpr (U8) {
-      stage_q(reinterpret_cast<float*>(kx), threadIdx.x, kPad, mk, qry[0], qmy[0], part + 0 * kQSums);
-      stage_q(reinterpret_cast<float*>(vx), threadIdx.x, kPad, mv, qry[1], qmy[1], part + 1 * kQSums);
-      stage_q(reinterpret_cast<float*>(rx), threadIdx.x, kPad, mr, qry[2], qmy[2], part + 2 * kQSums);
+      stage_xr(reinterpret_cast<float*>(kx), threadIdx.x, kPad, mk, qry[0]);
+      stage_xr(reinterpret_cast<float*>(vx), threadIdx.x, kPad, mv, qry[1]);
+      stage_xr(reinterpret_cast<float*>(rx), threadIdx.x, kPad, mr, qry[2]);
     } else {
       reinterpret_cast<h8*>(kx)[threadIdx.x] = mk;
       reinterpret_cast<h8*>(vx)[threadIdx.x] = mv;
@@ -459,11 +468,18 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
   zero_pad<U8>(kx, nchunk, kPad);
   zero_pad<U8>(vx, nchunk, kPad);
   zero_pad<U8>(rx, nchunk, kPad);
-  if constexpr (U8) publish_qsums(part, 3 * kQSums, qred);
   __syncthreads();
   load3_part(cur, c0 < c1 ? c0 : C - 1, c0 < c1, JH{}, JN{});  // the rest of the first channel's rows
   float qt[3 * kQSums];
   if constexpr (U8) {
+    // Sx and Smy of the three vectors are needed only when a row is finished: they are summed here, behind the
+    // barrier that releases the staged vectors and behind the last row requests, while the rows are on their way
+    // (every thread reaches both barriers; a thread without a group adds zeros).
+    sum_q(mk, qmy[0], part + 0 * kQSums);
+    sum_q(mv, qmy[1], part + 1 * kQSums);
+    sum_q(mr, qmy[2], part + 2 * kQSums);
+    publish_qsums(part, 3 * kQSums, qred);
+    __syncthreads();
     const float tv = gather_qsums(3 * kQSums, qred);
 #pragma unroll
     for (int i = 0; i < 3 * kQSums; i++) qt[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tv), i));
@@ -789,10 +805,14 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   request_ops(mA);
 
   // ---- prologue: stage the activation vector(s) in LDS ----
-  {
-    float part[kMaxSeg * kQSums];
+  // uint8: Sx and Smy of every staged vector are needed only when a row is finished.  They are summed behind the
+  // barrier that releases the staged vectors and behind the last row requests (below), from the values each thread
+  // keeps in `qx`, while the rows are on their way.
+  float part[kMaxSeg * kQSums];
 #pragma unroll
-    for (int i = 0; i < kMaxSeg * kQSums; i++) part[i] = 0.f;
+  for (int i = 0; i < kMaxSeg * kQSums; i++) part[i] = 0.f;
+  h8 qx[kMaxSeg] = {};
+  {
     if constexpr (PRO == P_COPY) {
 #pragma unroll
       for (int p = 0; p < kCopyPasses; p++) {
@@ -866,7 +886,8 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
                   if (a.seg[i].vec == j) mx8 = mixv[j];
                 x = mix8(ln.xx, sxv, mx8);
               }
-              stage_q(reinterpret_cast<float*>(vec_at(i)), threadIdx.x, kPad, x, qry[i], qmy[i], part + i * kQSums);
+              stage_xr(reinterpret_cast<float*>(vec_at(i)), threadIdx.x, kPad, x, qry[i]);
+              qx[i] = x;
             }
           }
         }
@@ -874,12 +895,23 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       }
     }
     for (int i = 0; i < (U8 ? a.nseg : a.nvec); i++) zero_pad<U8>(vec_at(i), nchunk, kPad);
-    if constexpr (U8) publish_qsums(part, a.nseg * kQSums, qred);
+    // (a ready vector is staged within a fraction of a microsecond and its rows are few: there the sums stay ahead of the barrier)
+    if constexpr (U8 && PRO == P_COPY) publish_qsums(part, a.nseg * kQSums, qred);
     __syncthreads();
-    if constexpr (U8) qtv = gather_qsums(a.nseg * kQSums, qred);
   }
   // ---- the rest of the first batch ----
   request_rows(A, whA, JH{}, JN{});
+  if constexpr (U8) {
+    // (every thread reaches the second barrier; threads without a group add zeros; the wide layernorm has summed already)
+    if constexpr (PRO != P_COPY) {
+#pragma unroll
+      for (int i = 0; i < kMaxSeg; i++)
+        if (i < a.nseg) sum_q(qx[i], qmy[i], part + i * kQSums);
+      publish_qsums(part, a.nseg * kQSums, qred);
+      __syncthreads();
+    }
+    qtv = gather_qsums(a.nseg * kQSums, qred);
+  }
 
   if constexpr (!MULTI) {
     consume(A, mA);  // the host guarantees at most one batch per wave
