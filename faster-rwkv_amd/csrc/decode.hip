@@ -505,24 +505,33 @@ __global__ __launch_bounds__(kThreads) void att_front_v4_kernel(AttFrontV4 a) {
       v = finish_q(v, (float)st.qrx[1], (float)st.qmx[1], qt[2], qt[3]);
       rr = finish_q(rr, (float)st.qrx[2], (float)st.qmx[2], qt[4], qt[5]);
     }
+    // kernels/cuda/att.cu:30-62 (WkvForwardOne), r already passed through sigmoid (:203).
+    // The update is a chain of five exponentials and two quotients on one channel's scalars, at the very end of
+    // the launch.  Every lane holds k, v and the r sum, so lanes 0..4 evaluate the five exponentials in one
+    // call and lanes 0, 1 the two quotients in one division: the same functions on the same arguments (the
+    // results are those of the serial chain bit for bit), a third of its instructions in sequence.
+    const h1 rh = (h1)rr;
+    const float pp_ = st.pp, aa_ = st.aa, bb_ = st.bb;
+    const float ww = st.tf + k;
+    const float p1 = (pp_ > ww) ? pp_ : ww;
+    const float ww2 = st.td + pp_;
+    const float p2 = (ww2 > k) ? ww2 : k;
+    const float arg = lane == 0 ? pp_ - p1 : lane == 1 ? ww - p1 : lane == 2 ? ww2 - p2 : lane == 3 ? k - p2 : -(float)rh;
+    const float e = expf(arg);
+    auto lane_of = [](float x, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), l)); };
+    const float e1 = lane_of(e, 0), e2 = lane_of(e, 1), e1n = lane_of(e, 2), e2n = lane_of(e, 3), es = lane_of(e, 4);
+    const float num = lane == 0 ? (e1 * aa_ + e2 * v) : 1.0f;
+    const float den = lane == 0 ? (e1 * bb_ + e2) : (1.0f + es);
+    const float quo = num / den;
+    const float wkv = lane_of(quo, 0), s32 = lane_of(quo, 1);  // s32 = 1 / (1 + exp(-r)): sigmoid_h_fast's value
     if (lane == 0) {
-      // kernels/cuda/att.cu:30-62 (WkvForwardOne), r already passed through sigmoid (:203)
-      const h1 r = sigmoid_h((h1)rr);
-      float ww = st.tf + k;
-      const float pp_ = st.pp;
-      float p_ = (pp_ > ww) ? pp_ : ww;
-      float e1 = expf(pp_ - p_);
-      float e2 = expf(ww - p_);
-      const float aa_ = st.aa, bb_ = st.bb;
-      const float wkv = (e1 * aa_ + e2 * v) / (e1 * bb_ + e2);
+      const uint32_t frac = __float_as_uint(s32) & 0x1FFFu;
+      const bool safe = s32 > 1e-4f && (frac < 0x1000u - 64u || frac > 0x1000u + 64u);
+      const h1 r = safe ? (h1)s32 : sigmoid_h_exact(rh);
       a.rwkv_out[n] = r * (h1)wkv;
-      ww = st.td + pp_;
-      p_ = (ww > k) ? ww : k;
-      e1 = expf(ww - p_);
-      e2 = expf(k - p_);
-      a.aa_out[n] = e1 * aa_ + e2 * v;
-      a.bb_out[n] = e1 * bb_ + e2;
-      a.pp_out[n] = p_;
+      a.aa_out[n] = e1n * aa_ + e2n * v;
+      a.bb_out[n] = e1n * bb_ + e2n;
+      a.pp_out[n] = p2;
     }
   };
 
