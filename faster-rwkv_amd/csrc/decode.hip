@@ -811,7 +811,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // ---- first batch of rows: the chunks that go out ahead of the prologue (see RowBatch::kHead) ----
   RowBatch<R, NCH, U8> A;
   request_rows(A, whA, J0{}, JH{});
-  request_ops(mA);
+  if constexpr (!U8) request_ops(mA);
 
   // ---- prologue: stage the activation vector(s) in LDS ----
   // uint8: Sx and Smy of every staged vector are needed only when a row is finished.  They are summed behind the
@@ -910,6 +910,10 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   }
   // ---- the rest of the first batch ----
   request_rows(A, whA, JH{}, JN{});
+  // uint8: the per-row operands (two more 2-byte loads per lane: rx, mx) go out behind all rows of the batch; ahead of
+  // the prologue they cost these launches more than the memory latency they save at the end (decode kernels 0.588 ->
+  // 0.583 ms per token; binary16, with at most two such loads, the other way round: 0.662 -> 0.669).
+  if constexpr (U8) request_ops(mA);
   if constexpr (U8) {
     // (every thread reaches the second barrier; threads without a group add zeros; the wide layernorm has summed already)
     if constexpr (PRO != P_COPY) {
