@@ -343,6 +343,26 @@ class Model:
     def reset(self):
         self._chk(self._h.fr_model_reset(self._m))
 
+    # The names of the reference's Python wrapper (python/fr_python.cpp:48-56, python/fasterrwkv/__init__.py:19-25):
+    # model(ids) -> logits as a numpy array, model.reset_states(), model.states().
+    __call__ = run
+    reset_states = reset
+
+    def states(self):
+        """Model::states() copied to the host: per layer a list of numpy arrays (RWKV-4: [C] act, three [C] fp32,
+        [C] act; RWKV-5.x: [C] act, [H, S, S] fp32, [C] act -- model.cpp:145-177)."""
+        v5 = self.n_head > 0  # RWKV-4 models have no heads
+        out = []
+        for l in range(self.n_layer):
+            if v5:
+                S = self.n_embd // self.n_head
+                out.append([self.state(l, 0, np.float16), self.state(l, 1, np.float32).reshape(self.n_head, S, S),
+                            self.state(l, 2, np.float16)])
+            else:
+                out.append([self.state(l, 0, np.float16)] + [self.state(l, j, np.float32) for j in (1, 2, 3)]
+                           + [self.state(l, 4, np.float16)])
+        return out
+
     def save_state(self, path):
         self._chk(self._h.fr_model_save_state(self._m, path.encode()))
 
@@ -416,6 +436,8 @@ class Sampler:
         if r < 0:
             raise FrhipError(self._h.fr_last_error().decode())
         return r
+
+    __call__ = sample  # python/fasterrwkv/__init__.py:25
 
     def __del__(self):
         if getattr(self, "_s", None):

@@ -51,6 +51,23 @@ def test_model_run_matches_oracle_over_128_greedy_steps(model_files, strategy):
     m.close()
 
 
+def test_python_names_of_the_reference_wrapper(model_files):
+    """python/fr_python.cpp:48-56, python/fasterrwkv/__init__.py:19-25: model(ids) -> numpy logits,
+    model.reset_states(), model.states(), sampler(logits, ...)."""
+    path, params, emb = model_files
+    m = fr.Model(path, "hip fp16")
+    a = m([5, 6, 7])
+    st = m.states()
+    assert len(st) == L_ and [x.shape for x in st[0]] == [(C_,)] * 5
+    assert st[0][0].dtype == np.float16 and st[0][1].dtype == np.float32 and np.abs(st[0][1]).max() > 0
+    m.reset_states()
+    assert np.all(m.states()[3][1] == 0) and np.all(m.states()[3][3] == np.float32(-1e30))  # model.cpp:152-160
+    assert np.array_equal(m([5, 6, 7]), a)
+    smp = fr.Sampler(seed=3)
+    assert smp(a, 1.0, 1, 0.0) == int(np.argmax(a))  # top_k = 1 is the arg-max
+    m.close()
+
+
 def test_fused_graph_path_equals_operator_by_operator_path(model_files):
     path, _, _ = model_files
     ids = [3, 1000, 77, 77, 4095, 0, 9]
