@@ -1081,7 +1081,6 @@ __global__ __launch_bounds__(kThreads) void rows_sliced_kernel(RowsArgs a, Slice
   const int lane = threadIdx.x & (kWave - 1);
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const Seg& sg = a.seg[0];
-  const int N = sg.w.N;
   float* partials = reinterpret_cast<float*>(smem + g.part_offset);
   int r0, r1;  // this workgroup's rows
   split_even(g.rows, blockIdx.x, r0, r1);

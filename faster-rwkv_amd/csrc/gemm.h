@@ -48,7 +48,7 @@ struct GemmArgs {
 // partial: optional fp32 scratch of max_split slices of partial_stride floats (>= M * N each) for splitting K.
 int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq = nullptr, float* partial = nullptr,
                 size_t partial_stride = 0, int max_split = 0);
-constexpr int kDequantRows = 192;
+constexpr int kDequantRows = FRHIP_SEQ_EXPAND_ROWS;
 // uint8 [N][K] -> binary16 [N][K] with the frozen formula (ops.hip)
 int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,
                      hipStream_t st);

@@ -22,12 +22,22 @@ frhip_stream stream();
 struct PackedWeight {
   frhip_weight desc{};
   std::vector<Tensor> owners;  // device buffers: data, then mx rx my ry for uint8
+  // uint8 only, made on first use by find_seq_weight: the binary16 image [N, K] of the weight
+  // (frhip_dequant_u8) and its description.  Freed with the weight.
+  Tensor image;
+  frhip_weight image_desc{};
 };
 
 void register_weight(const void *data_ptr, std::shared_ptr<PackedWeight> w);
 void unregister_weight(const void *data_ptr);
 // nullptr when `t` is not a packed weight.
 const frhip_weight *find_weight(const Tensor &t);
+// The description to hand to a product over `rows` rows of activations.  The same as
+// find_weight unless FR_HIP_SEQ_IMAGE=1 is set, the weight is uint8 and rows >=
+// FRHIP_SEQ_EXPAND_ROWS: then the weight's binary16 image, expanded once and kept (2 more
+// bytes per weight for as long as the model lives) instead of once per call into the
+// operator's workspace.  Both ways multiply by the same w^, so the results are the same bits.
+const frhip_weight *find_seq_weight(const Tensor &t, int rows);
 
 // Upload a host matrix in the reference's [K, N] layout and pack it for the kernels.
 // `dtype` kFloat16: src is binary16.  kInt8: src is binary16 and is quantised on the host

@@ -376,7 +376,7 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
     pi += 7;
     if ((i + 1) % 6 == 0) scalar_div_(x, 2);
   }
-  const frhip_weight *hw = find_weight(p[pi + 2]);
+  const frhip_weight *hw = find_seq_weight(p[pi + 2], full_output ? T : 1);
   RV_CHECK(hw != nullptr);
   if (full_output) {
     // every row -> ln_out -> head -> fp32 [T, V] (model_forward_seq.cpp:173-178 without the slice)

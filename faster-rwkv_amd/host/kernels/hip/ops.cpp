@@ -21,8 +21,9 @@ int to_frhip_dtype(DType d) {
 
 // Packed description of a weight tensor.  A tensor that did not come from init_model
 // (a plain [K, N] binary16 matrix on the device) is packed on the fly into `tmp`.
-const frhip_weight *weight_of(const Tensor &w, frhip_weight &tmp_desc, Tensor &tmp) {
-  if (const frhip_weight *p = find_weight(w)) return p;
+// `rows`: rows of activations the product will have (1 for the one-token operators).
+const frhip_weight *weight_of(const Tensor &w, frhip_weight &tmp_desc, Tensor &tmp, int rows = 1) {
+  if (const frhip_weight *p = find_seq_weight(w, rows)) return p;
   RV_CHECK(w.shape().size() == 2 && w.dtype() == DType::kFloat16)
       << "matmul on hip: right operand must be a packed weight or a 2-D fp16 tensor";
   const int K = static_cast<int>(w.size(0)), N = static_cast<int>(w.size(1));
@@ -95,7 +96,7 @@ Tensor matmul(const Tensor &a, const Tensor &b) {
   RV_CHECK(a.size(-1) == b.size(0)) << "matmul: " << shape_str(a.shape()) << " x " << shape_str(b.shape());
   frhip_weight tmp_desc;
   Tensor tmp;
-  const frhip_weight *w = weight_of(b, tmp_desc, tmp);
+  const frhip_weight *w = weight_of(b, tmp_desc, tmp, a.sizes().size() == 2 ? static_cast<int>(a.size(0)) : 1);
   if (a.sizes().size() == 2) {  // matrix x matrix (matmul.cpp:110-121): the MFMA product
     const int T = static_cast<int>(a.size(0));
     Tensor c = Tensor::Empty({a.size(0), b.size(1)}, a.dtype(), Device::kHIP);
@@ -317,7 +318,7 @@ std::tuple<Tensor, Tensor> ffn_seq(const Tensor &x, const Tensor &sx, const Tens
   const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1)), F = static_cast<int>(kw.size(1));
   frhip_weight d[3];
   Tensor tmp[3];
-  const frhip_weight *w[3] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2])};
+  const frhip_weight *w[3] = {weight_of(kw, d[0], tmp[0], T), weight_of(vw, d[1], tmp[1], T), weight_of(rw, d[2], tmp[2], T)};
   Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
   Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
   Tensor ws = seq_workspace(T, C, F);
@@ -336,8 +337,8 @@ att_seq(const Tensor &x, const Tensor &sx, const Tensor &aa, const Tensor &bb, c
   const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1));
   frhip_weight d[4];
   Tensor tmp[4];
-  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
-                              weight_of(ow, d[3], tmp[3])};
+  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0], T), weight_of(vw, d[1], tmp[1], T), weight_of(rw, d[2], tmp[2], T),
+                              weight_of(ow, d[3], tmp[3], T)};
   Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
   Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
   Tensor t1 = Tensor::Empty(aa.sizes(), DType::kFloat32, Device::kHIP);
@@ -365,8 +366,8 @@ att_seq_v5_2(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &l
   const int H = static_cast<int>(t_decay.size(0));
   frhip_weight d[5];
   Tensor tmp[5];
-  const frhip_weight *w[5] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
-                              weight_of(gw, d[3], tmp[3]), weight_of(ow, d[4], tmp[4])};
+  const frhip_weight *w[5] = {weight_of(kw, d[0], tmp[0], T), weight_of(vw, d[1], tmp[1], T), weight_of(rw, d[2], tmp[2], T),
+                              weight_of(gw, d[3], tmp[3], T), weight_of(ow, d[4], tmp[4], T)};
   Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
   Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
   Tensor s_out = Tensor::Empty(s.sizes(), DType::kFloat32, Device::kHIP);
@@ -391,8 +392,8 @@ att_seq_v5(const Tensor &x, const Tensor &sx, const Tensor &s, const Tensor &ln_
   RV_CHECK(t_decay.numel() == H && t_first.numel() == H) << "att_seq_v5: time_decay/time_first must hold one value per head";
   frhip_weight d[4];
   Tensor tmp[4];
-  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0]), weight_of(vw, d[1], tmp[1]), weight_of(rw, d[2], tmp[2]),
-                              weight_of(ow, d[3], tmp[3])};
+  const frhip_weight *w[4] = {weight_of(kw, d[0], tmp[0], T), weight_of(vw, d[1], tmp[1], T), weight_of(rw, d[2], tmp[2], T),
+                              weight_of(ow, d[3], tmp[3], T)};
   Tensor x_out = Tensor::Empty(x.sizes(), x.dtype(), Device::kHIP);
   Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
   Tensor s_out = Tensor::Empty(s.sizes(), DType::kFloat32, Device::kHIP);

@@ -51,6 +51,31 @@ const frhip_weight *find_weight(const Tensor &t) {
   return it == table().end() ? nullptr : &it->second->desc;
 }
 
+const frhip_weight *find_seq_weight(const Tensor &t, int rows) {
+  const char *e = std::getenv("FR_HIP_SEQ_IMAGE");  // read per call, like FR_HIP_GENERIC
+  const bool keep = e && std::atoi(e) != 0;
+  if (!keep || rows < FRHIP_SEQ_EXPAND_ROWS) return find_weight(t);
+  if (!t.defined() || t.device() != Device::kHIP) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto it = table().find(t.data_ptr());
+  if (it == table().end()) return nullptr;
+  PackedWeight &w = *it->second;
+  if (w.desc.dtype != FRHIP_U8) return &w.desc;
+  if (!w.image.defined()) {
+    // on the backend's stream, like every product that will read it
+    Tensor img = Tensor::Empty({static_cast<LengthType>(w.desc.N), static_cast<LengthType>(w.desc.K)}, DType::kFloat16,
+                               Device::kHIP);
+    FRHIP_CHECK(frhip_dequant_u8(&w.desc, img.data_ptr(), stream()));
+    w.image = img;
+    w.image_desc = frhip_weight{};
+    w.image_desc.data = w.image.data_ptr();
+    w.image_desc.K = w.desc.K;
+    w.image_desc.N = w.desc.N;
+    w.image_desc.dtype = FRHIP_F16;
+  }
+  return &w.image_desc;
+}
+
 static inline float h2f(uint16_t b) {
   float16 h;
   h.bits = b;

@@ -126,6 +126,41 @@ def test_seq_mode_equals_one_token_steps_and_oracle(model_files, strategy):
     m.close()
 
 
+@pytest.mark.parametrize("spec", ["v=4,L=3,C=512,F=2048,V=2048,seed=11", "v=5.2,L=3,C=512,F=1792,V=2048,H=8,seed=12"])
+@pytest.mark.parametrize("generic", [False, True])
+def test_kept_binary16_image_of_uint8_weights_gives_the_same_bits(spec, generic):
+    """FR_HIP_SEQ_IMAGE=1: prompts of FRHIP_SEQ_EXPAND_ROWS rows or more multiply the kept binary16
+    image of the uint8 weights instead of one expanded per call; w^ is the same, so logits (last
+    row and every row) and the state left behind are the same bits.  Shorter prompts and one-token
+    steps still read the codes."""
+    ids = [int(t) for t in np.random.default_rng(47).integers(0, 2048, 300)]
+
+    def run():
+        m = fr.Model("synthetic:" + spec, "hip int8")
+        out = [m.run(ids), m.run(ids[:250]), m.run(5), m.run(ids[:64]), m.run(6)]
+        m.reset()
+        out.append(m.run_full(ids[:200]))
+        out += [st for layer in m.states() for st in layer]
+        m.close()
+        return out
+
+    env = {"FR_HIP_SEQ_IMAGE": "1", **({"FR_HIP_GENERIC": "1"} if generic else {})}
+    saved = {k: os.environ.get(k) for k in env}
+    plain = None
+    try:
+        if generic:
+            os.environ["FR_HIP_GENERIC"] = "1"
+        plain = run()
+        os.environ.update(env)
+        kept = run()
+    finally:
+        for k, v in saved.items():
+            os.environ.pop(k, None) if v is None else os.environ.__setitem__(k, v)
+    assert len(plain) == len(kept)
+    for a, b in zip(plain, kept):
+        assert np.array_equal(a, b)
+
+
 def test_synthetic_model_and_cpp_greedy_loop():
     m = fr.Model("synthetic:v=4,L=2,C=256,F=1024,V=1024,seed=7", "hip int8")
     toks, secs = m.greedy(1, 16)
