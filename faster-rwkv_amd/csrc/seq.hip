@@ -366,6 +366,10 @@ __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
 // j = t % 64 and key rows i = (t / 64) * 16 .. +15 of the state (16 registers).
 // Output row t: y_j = sum_i r_i (u_i k_i v_j + s_ij), then groupnorm over the head's 64
 // values, rounding to half and the gate multiply (att_seq.cu:294-316, :406-411).
+// The scan over a prompt regroups the sums by chunk anyway, so its multiply-adds are fused (four
+// instructions per state element and step instead of seven); the one-token operator keeps the
+// separately rounded products and sums.  The partial sums of 16 steps wait in LDS for one round
+// of group norms shared by the four waves, instead of a barrier and one wave's group norm per step.
 // ---------------------------------------------------------------------------
 struct Wkv5Seq {
   int T, C, H, Lc, nchunk;
@@ -403,9 +407,7 @@ __global__ __launch_bounds__(256) void wkv5_local_kernel(Wkv5Seq a) {
 #pragma unroll
     for (int ii = 0; ii < 16; ii++) {
       const int i = ig * 16 + ii;
-      const float aij = kk[tt * S5 + i] * vj;
-      const float ws = wsh[i] * s[ii];
-      s[ii] = ws + aij;
+      s[ii] = __builtin_fmaf(wsh[i], s[ii], kk[tt * S5 + i] * vj);
     }
   }
   float* dst = a.loc + ((size_t)ch * a.H + h) * S5 * S5;
@@ -413,8 +415,9 @@ __global__ __launch_bounds__(256) void wkv5_local_kernel(Wkv5Seq a) {
   for (int ii = 0; ii < 16; ii++) dst[(ig * 16 + ii) * S5 + j] = s[ii];
 }
 
-// The serial pass over the chunks, one state element per thread; the chunks' local end states are
-// read eight at a time ahead of the recurrence.
+// The serial pass over the chunks, one state element per thread.  The decay of the incoming state
+// over a whole chunk is one multiplication by w^Lc (formed once by repeated multiplication), and the
+// chunks' local end states are read eight at a time, the next eight while these are consumed.
 __global__ __launch_bounds__(256) void wkv5_carry_kernel(Wkv5Seq a) {
   const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;  // element of [H][64][64]
   const size_t per = (size_t)a.H * S5 * S5;
@@ -422,21 +425,28 @@ __global__ __launch_bounds__(256) void wkv5_carry_kernel(Wkv5Seq a) {
   constexpr int PF = 8;
   const int i = (int)((e / S5) % S5), h = (int)(e / (S5 * S5));
   const float w = a.w[a.uw_head ? h : h * S5 + i];
-  float s = a.s[e];
-  for (int ch0 = 0; ch0 < a.nchunk; ch0 += PF) {
-    float loc[PF];
+  float cur[PF], nxt[PF];
 #pragma unroll
-    for (int j = 0; j < PF; j++) loc[j] = a.loc[(size_t)(ch0 + j < a.nchunk ? ch0 + j : a.nchunk - 1) * per + e];
+  for (int j = 0; j < PF; j++) cur[j] = a.loc[(size_t)(j < a.nchunk ? j : a.nchunk - 1) * per + e];
+  float s = a.s[e];
+  float wl = 1.0f;  // w^Lc; the last chunk may be shorter, but nothing is carried out of it here
+  for (int q = 0; q < a.Lc; q++) wl *= w;
+  for (int ch0 = 0; ch0 < a.nchunk; ch0 += PF) {
+#pragma unroll
+    for (int j = 0; j < PF; j++) {
+      const int ch = ch0 + PF + j;
+      nxt[j] = a.loc[(size_t)(ch < a.nchunk ? ch : a.nchunk - 1) * per + e];
+    }
 #pragma unroll
     for (int j = 0; j < PF; j++) {
       const int ch = ch0 + j;
       if (ch < a.nchunk) {
         a.sin[(size_t)ch * per + e] = s;
-        const int len = min(a.Lc, a.T - ch * a.Lc);
-        for (int q = 0; q < len; q++) s = w * s;  // decay of the incoming state over the chunk
-        s = s + loc[j];
+        s = __builtin_fmaf(wl, s, cur[j]);
       }
     }
+#pragma unroll
+    for (int j = 0; j < PF; j++) cur[j] = nxt[j];
   }
 }
 
@@ -446,7 +456,8 @@ __global__ __launch_bounds__(256) void wkv5_apply_kernel(Wkv5Seq a) {
   float* kk = rr + a.Lc * S5;
   float* vv = kk + a.Lc * S5;
   __shared__ float wsh[S5], ush[S5];
-  __shared__ float part[2][4][S5];
+  constexpr int kGroup = 16;  // steps whose partial sums wait in LDS for one round of group norms
+  __shared__ float part[kGroup][4][S5];
   const int h = blockIdx.x, ch = blockIdx.y, t = threadIdx.x, j = t & 63, ig = t >> 6;
   const int t0 = ch * a.Lc, len = min(a.Lc, a.T - t0);
   for (int e = t; e < len * S5; e += 256) {
@@ -463,38 +474,44 @@ __global__ __launch_bounds__(256) void wkv5_apply_kernel(Wkv5Seq a) {
   float s[16];
 #pragma unroll
   for (int ii = 0; ii < 16; ii++) s[ii] = src[(ig * 16 + ii) * S5 + j];
-  float gw = 0.f, gb = 0.f;
-  if (t < S5) {
-    gw = a.lx_w[h * S5 + t];
-    gb = a.lx_b[h * S5 + t];
-  }
+  const float gw = a.lx_w[h * S5 + j], gb = a.lx_b[h * S5 + j];
   __syncthreads();
-  for (int tt = 0; tt < len; tt++) {
-    const float vj = vv[tt * S5 + j];
-    float acc = 0.f;
+  float wr[16], ur[16];
 #pragma unroll
-    for (int ii = 0; ii < 16; ii++) {
-      const int i = ig * 16 + ii;
-      const float aij = kk[tt * S5 + i] * vj;
-      const float ua = ush[i] * aij;
-      const float tmp = ua + s[ii];
-      const float ws = wsh[i] * s[ii];
-      s[ii] = ws + aij;
-      acc += rr[tt * S5 + i] * tmp;
+  for (int ii = 0; ii < 16; ii++) {
+    wr[ii] = wsh[ig * 16 + ii];
+    ur[ii] = ush[ig * 16 + ii];
+  }
+  for (int tb = 0; tb < len; tb += kGroup) {
+    const int n = min(kGroup, len - tb);
+    for (int q = 0; q < n; q++) {
+      const int tt = tb + q;
+      const float vj = vv[tt * S5 + j];
+      float acc = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < 16; ii++) {
+        const int i = ig * 16 + ii;
+        const float aij = kk[tt * S5 + i] * vj;
+        const float tmp = __builtin_fmaf(ur[ii], aij, s[ii]);
+        s[ii] = __builtin_fmaf(wr[ii], s[ii], aij);
+        acc = __builtin_fmaf(rr[tt * S5 + i], tmp, acc);
+      }
+      part[q][ig][j] = acc;
     }
-    part[tt & 1][ig][j] = acc;
-    __syncthreads();  // the other half of `part` is free again: its readers passed this barrier a step ago
-    if (t < S5) {
-      const float o = ((part[tt & 1][0][t] + part[tt & 1][1][t]) + part[tt & 1][2][t]) + part[tt & 1][3][t];
+    __syncthreads();
+    // wave ig: the group norms of steps ig, ig + 4, ... of this round
+    for (int q = ig; q < n; q += 4) {
+      const float o = ((part[q][0][j] + part[q][1][j]) + part[q][2][j]) + part[q][3][j];
       const float mean = wave_sum(o) / (float)S5;
       const float d = o - mean;
       float var = wave_sum(d * d) / (float)S5;
       var = var > 0.f ? var : 0.f;
       const float inv = 1.0f / sqrtf(var + 1e-5f);
       const float y = d * inv * gw + gb;
-      const size_t oi = (size_t)(t0 + tt) * a.C + h * S5 + t;
+      const size_t oi = (size_t)(t0 + tb + q) * a.C + h * S5 + j;
       a.gated[oi] = a.g ? (h1)y * a.g[oi] : (h1)y;
     }
+    __syncthreads();  // `part` is free for the next round
   }
   if (ch == a.nchunk - 1) {
     float* dst = a.s_out + (size_t)h * S5 * S5;
