@@ -107,6 +107,48 @@ __global__ __launch_bounds__(256) void embed_ring_kernel(const unsigned char* __
   for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x) dst[i] = src[i];
 }
 
+// Token feed of a greedy loop that stays on the device: the token of this step is the arg-max of the
+// previous step's logits, taken from that step's per-slice {value, index} pairs (greater value, then
+// smaller index; index n_rows or beyond, i.e. no finite maximum, gives token 0: the host's rule).
+// The token goes to ids[*counter % ids_len] for the host to read later, *counter advances, and the
+// token's row of `table` is copied to `out`.
+__global__ __launch_bounds__(256) void embed_argmax_kernel(const unsigned char* __restrict__ table, int n_rows,
+                                                           int row_bytes, const float* pairs, int npairs, int32_t* ids,
+                                                           int ids_len, uint32_t* counter, unsigned char* __restrict__ out) {
+  __shared__ int row;
+  if (threadIdx.x < 64) {
+    float best = -INFINITY;
+    int idx = n_rows;
+    for (int b = threadIdx.x; b < npairs; b += 64) {
+      const float v = pairs[2 * b];
+      const int i = reinterpret_cast<const int32_t*>(pairs)[2 * b + 1];
+      if (v > best || (v == best && i < idx)) {
+        best = v;
+        idx = i;
+      }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off);
+      const int oi = __shfl_xor(idx, off);
+      if (ov > best || (ov == best && oi < idx)) {
+        best = ov;
+        idx = oi;
+      }
+    }
+    if (threadIdx.x == 0) {
+      const int id = (idx >= 0 && idx < n_rows) ? idx : 0;
+      const uint32_t c = *counter;
+      ids[c % (uint32_t)ids_len] = id;
+      *counter = c + 1;
+      row = id;
+    }
+  }
+  __syncthreads();
+  const u32x4* src = reinterpret_cast<const u32x4*>(table + (size_t)row * row_bytes);
+  u32x4* dst = reinterpret_cast<u32x4*>(out);
+  for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x) dst[i] = src[i];
+}
+
 // [K][N] -> [N][K] through a 64x64 LDS tile (+1 padding against bank conflicts).
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst, int K, int N) {
@@ -558,6 +600,16 @@ int frhip_embed_ring(const void* table, int n_rows, int row_bytes, const int32_t
   hipLaunchKernelGGL(embed_ring_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(s),
                      (const unsigned char*)table, n_rows, row_bytes, ring, ring_len, counter_dev, (unsigned char*)out);
   return check_launch("embed_ring");
+}
+
+int frhip_embed_argmax(const void* table, int n_rows, int row_bytes, const void* pairs, int npairs, int32_t* ids,
+                       int ids_len, uint32_t* counter_dev, void* out, frhip_stream s) {
+  if (!table || !pairs || !ids || !counter_dev || !out) return set_error(FRHIP_EINVAL, "embed_argmax: null pointer");
+  if (n_rows <= 0 || npairs <= 0 || ids_len <= 0 || row_bytes <= 0 || row_bytes % 16 != 0)
+    return set_error(FRHIP_ESHAPE, "embed_argmax: row_bytes must be a positive multiple of 16");
+  hipLaunchKernelGGL(embed_argmax_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(s), (const unsigned char*)table,
+                     n_rows, row_bytes, (const float*)pairs, npairs, ids, ids_len, counter_dev, (unsigned char*)out);
+  return check_launch("embed_argmax");
 }
 
 int frhip_pack_transpose(const void* src, void* dst, int K, int N, int elem_bytes, frhip_stream s) {

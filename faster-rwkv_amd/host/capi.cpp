@@ -198,14 +198,17 @@ int fr_model_get_state(void *m, int layer, int index, void *out, int capacity) {
 
 // Greedy decoding as chat.cpp:56-92 does with top_k = 1: feed `first_id`, take the argmax of
 // the returned (host) logits, feed it back.  out_ids receives `steps` tokens.  Returns the
-// wall time of the loop in microseconds (>= 0) or -1.
+// wall time of the loop in microseconds (>= 0) or -1.  On the fused hip path the choice of the
+// token stays on the device and the host waits once per batch of steps (hip::GreedyDecode).
 long long fr_greedy_decode(void *m, int first_id, int steps, int *out_ids) {
   long long us = -1;
   guarded([&]() {
     auto *model = static_cast<rwkv::Model *>(m);
     int id = first_id;
     const auto t0 = std::chrono::steady_clock::now();
-    for (int i = 0; i < steps; i++) {
+    // the fused hip path keeps the whole loop on the device (FR_HIP_GREEDY_ON_HOST=1: token by token, as below)
+    const bool chained = rwkv::hip::GreedyDecode(model, first_id, steps, out_ids);
+    for (int i = 0; i < steps && !chained; i++) {
       rwkv::Tensor out = model->Run(id);
       // the fused hip path has taken the argmax on the device (first index on ties, like argmax())
       if (!rwkv::hip::device_argmax(model, out, &id))

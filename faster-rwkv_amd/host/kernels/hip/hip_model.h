@@ -24,6 +24,8 @@ struct ModelExtra {
 
 std::shared_ptr<ModelExtra> extra_of(Model *model);
 bool device_argmax(Model *model, const Tensor &logits, int *id);
+// `steps` greedy tokens from `first_id` with the token choice left on the device (model_forward.cpp).
+bool GreedyDecode(Model *model, int first_id, int steps, int *out_ids, Tensor *last_logits = nullptr);
 
 // Defined in kernels/default/model_forward.cpp
 }  // namespace hip

@@ -11,8 +11,13 @@
 // (Model::states()) is kept as views of these buffers; states assigned from outside
 // (ResetStates, LoadStateFile, set_states) are copied in on the next call.
 //
+// A greedy loop (GreedyDecode, behind fr_greedy_decode) does not need the host between two tokens:
+// a second set of graphs starts with a kernel that picks the token from the arg-max pairs the previous
+// token left behind, so the tokens are queued back to back and the host waits once per batch.
+//
 // FR_HIP_GENERIC=1 selects the operator-by-operator loops (one token and seq mode) instead; FR_HIP_NO_GRAPH=1 keeps
 // the fused path but launches eagerly.
+#include <algorithm>
 #include <cstdlib>
 #include <cmath>
 #include <cstring>
@@ -50,12 +55,23 @@ struct DecodePlan {
   size_t n_state() const { return v5 ? 3 : 5; }
   int parity = 0;                             // which ping-pong side holds the current shift states
   frhip_graph graph[2] = {nullptr, nullptr};
+  // greedy loop kept on the device (GreedyDecode): the same token, but its first kernel takes the token
+  // from the previous step's arg-max pairs and notes it in `chain_ids` (pinned) for the host
+  static constexpr int kChainIds = 1024;
+  frhip_graph chain[2] = {nullptr, nullptr};
+  frhip_graph chain_block = nullptr;  // chain_block_len (even) chained tokens starting on parity 0, as one graph
+  int chain_block_len = 2;            // FR_HIP_CHAIN_BLOCK: 2 measured best (4, 8: 0.7 % slower; 16, 32: 1.5-3 % slower)
+  int32_t *chain_ids = nullptr;
   bool use_graph = true;
   bool owned_logits = false;  // FR_HIP_OWNED_LOGITS: Run() returns a tensor of its own instead of a view of the pinned ring
   ~DecodePlan() {
     for (auto g : graph)
       if (g) frhip_graph_destroy(g);
+    for (auto g : chain)
+      if (g) frhip_graph_destroy(g);
+    if (chain_block) frhip_graph_destroy(chain_block);
     if (ring) frhip_host_free(ring);
+    if (chain_ids) frhip_host_free(chain_ids);
     for (auto h : logits_host)
       if (h) frhip_host_free(h);
   }
@@ -101,6 +117,8 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   void *h = nullptr;
   FRHIP_CHECK(frhip_host_malloc(&h, sizeof(int32_t) * DecodePlan::kRing));
   p->ring = static_cast<int32_t *>(h);
+  FRHIP_CHECK(frhip_host_malloc(&h, sizeof(int32_t) * DecodePlan::kChainIds));
+  p->chain_ids = static_cast<int32_t *>(h);
   for (auto &lh : p->logits_host) {
     FRHIP_CHECK(frhip_host_malloc(&h, sizeof(float) * (static_cast<size_t>(p->n_logits) + 2 * DecodePlan::kArgmaxBlocks)));
     lh = static_cast<float *>(h);
@@ -108,6 +126,7 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   alloc_state_buffers(*p);
   p->use_graph = std::getenv("FR_HIP_NO_GRAPH") == nullptr;  // fixed when the model first runs
   p->owned_logits = std::getenv("FR_HIP_OWNED_LOGITS") != nullptr;
+  if (const char *e = std::getenv("FR_HIP_CHAIN_BLOCK")) p->chain_block_len = std::atoi(e) / 2 * 2;  // 0: token by token
   return p;
 }
 
@@ -144,10 +163,13 @@ static void detach_if_snapshotted(Model *model, DecodePlan &p) {
       if (st[l][j].shares_storage_with(src)) st[l][j] = dst;
     }
   FRHIP_CHECK(frhip_stream_sync(stream()));
-  for (auto &g : p.graph) {
-    if (g) frhip_graph_destroy(g);
-    g = nullptr;
-  }
+  for (auto *set : {p.graph, p.chain})
+    for (int i = 0; i < 2; i++) {
+      if (set[i]) frhip_graph_destroy(set[i]);
+      set[i] = nullptr;
+    }
+  if (p.chain_block) frhip_graph_destroy(p.chain_block);
+  p.chain_block = nullptr;
 }
 
 // Bring states assigned from outside into the plan's buffers and rebind the model's
@@ -170,13 +192,20 @@ static void adopt_states(Model *model, DecodePlan &p) {
   }
 }
 
-static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
+// `chained`: the token comes from the arg-max pairs the previous step left behind its logits
+// (that step ran on the other parity) instead of from the host's ring.
+static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chained = false) {
   const auto &P = model->_params;
   frhip_stream s = stream();
   const int C = p.C, F = p.F;
   const int cur = p.parity, nxt = 1 - p.parity;
-  FRHIP_CHECK(frhip_embed_ring(ex.emb_table.data_ptr(), p.V, 2 * C, p.ring, DecodePlan::kRing,
-                               reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
+  if (chained)
+    FRHIP_CHECK(frhip_embed_argmax(ex.emb_table.data_ptr(), p.V, 2 * C, p.logits_host[nxt] + p.n_logits,
+                                   DecodePlan::kArgmaxBlocks, p.chain_ids, DecodePlan::kChainIds,
+                                   reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
+  else
+    FRHIP_CHECK(frhip_embed_ring(ex.emb_table.data_ptr(), p.V, 2 * C, p.ring, DecodePlan::kRing,
+                                 reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
   size_t pi = 0;
   for (int l = 0; l < p.L && p.v50; l++) {
     const frhip_weight *kw = find_weight(P[pi + 9]), *vw = find_weight(P[pi + 10]), *rw = find_weight(P[pi + 11]),
@@ -247,6 +276,83 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p) {
                                       DecodePlan::kArgmaxBlocks, s));
 }
 
+// Replays (capturing it first, if need be) the graph of one token on the current parity and moves the
+// plan on to the next token; does not wait.
+static void launch_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chained) {
+  frhip_stream s = stream();
+  const int cur = p.parity;
+  if (!p.use_graph) {
+    issue_token(model, ex, p, chained);
+  } else {
+    frhip_graph &g = chained ? p.chain[cur] : p.graph[cur];
+    if (!g) {
+      FRHIP_CHECK(frhip_graph_begin(s));
+      try {
+        issue_token(model, ex, p, chained);
+      } catch (...) {
+        frhip_graph dead = nullptr;
+        frhip_graph_end(s, &dead);
+        if (dead) frhip_graph_destroy(dead);
+        throw;
+      }
+      FRHIP_CHECK(frhip_graph_end(s, &g));
+    }
+    FRHIP_CHECK(frhip_graph_launch(g, s));
+  }
+  p.fed++;  // the device counter advances when the first kernel of the step runs
+  p.parity = 1 - cur;
+}
+
+// chain_block_len chained tokens in one graph (the gap between two graph launches on a stream is paid
+// once per block instead of once per token).  The plan must be on parity 0; it is again afterwards.
+static void launch_chain_block(Model *model, ModelExtra &ex, DecodePlan &p) {
+  frhip_stream s = stream();
+  RV_CHECK(p.parity == 0 && p.chain_block_len % 2 == 0);
+  if (!p.chain_block) {
+    FRHIP_CHECK(frhip_graph_begin(s));
+    try {
+      for (int k = 0; k < p.chain_block_len; k++) {
+        issue_token(model, ex, p, true);
+        p.parity = 1 - p.parity;
+      }
+    } catch (...) {
+      p.parity = 0;
+      frhip_graph dead = nullptr;
+      frhip_graph_end(s, &dead);
+      if (dead) frhip_graph_destroy(dead);
+      throw;
+    }
+    FRHIP_CHECK(frhip_graph_end(s, &p.chain_block));
+  }
+  FRHIP_CHECK(frhip_graph_launch(p.chain_block, s));
+  p.fed += p.chain_block_len;
+}
+
+// After the stream has been waited for: the model's state tensors follow the ping-pong side, and the
+// arg-max of the last token's logits (buffer `cur`) is finished on the host.
+static void settle(Model *model, ModelExtra &ex, DecodePlan &p, int cur) {
+  auto &st = model->states();
+  const size_t last = p.v5 ? 2 : 4;
+  for (int l = 0; l < p.L; l++) {
+    st[l][0] = p.view(p.parity, l, 0);
+    st[l][last] = p.view(p.parity, l, last);
+  }
+  // second step of the arg-max: greater value, then smaller index, over the per-slice pairs
+  const float *pairs = p.logits_host[cur] + p.n_logits;
+  float best = -INFINITY;
+  int32_t idx = p.n_logits;
+  for (int b = 0; b < DecodePlan::kArgmaxBlocks; b++) {
+    int32_t bi;
+    std::memcpy(&bi, pairs + 2 * b + 1, sizeof(bi));
+    if (pairs[2 * b] > best || (pairs[2 * b] == best && bi < idx)) {
+      best = pairs[2 * b];
+      idx = bi;
+    }
+  }
+  ex.last_argmax = idx < p.n_logits ? idx : 0;
+  ex.last_argmax_of = p.logits_host[cur];
+}
+
 Tensor ModelForward(Model *model, Device device, int id) {
   const bool generic = std::getenv("FR_HIP_GENERIC") != nullptr;  // read per call so that one process can compare both paths
   const std::string &ver = model->version();
@@ -257,55 +363,15 @@ Tensor ModelForward(Model *model, Device device, int id) {
   RV_CHECK(id >= 0 && id < p.V) << "token id " << id << " out of range";
   detach_if_snapshotted(model, p);
   adopt_states(model, p);
-  frhip_stream s = stream();
   // every call ends with a stream synchronisation, so the device has consumed all earlier slots
   p.ring[p.fed % DecodePlan::kRing] = id;
   const int cur = p.parity;
-  if (!p.use_graph) {
-    issue_token(model, *ex, p);
-  } else {
-    if (!p.graph[cur]) {
-      FRHIP_CHECK(frhip_graph_begin(s));
-      try {
-        issue_token(model, *ex, p);
-      } catch (...) {
-        frhip_graph g = nullptr;
-        frhip_graph_end(s, &g);
-        if (g) frhip_graph_destroy(g);
-        throw;
-      }
-      FRHIP_CHECK(frhip_graph_end(s, &p.graph[cur]));
-    }
-    FRHIP_CHECK(frhip_graph_launch(p.graph[cur], s));
-  }
-  p.fed++;  // the device counter advances when the first kernel of the step runs
-  p.parity = 1 - cur;
-  auto &st = model->states();
-  const size_t last = p.v5 ? 2 : 4;
-  for (int l = 0; l < p.L; l++) {
-    st[l][0] = p.view(p.parity, l, 0);
-    st[l][last] = p.view(p.parity, l, last);
-  }
+  launch_token(model, *ex, p, false);
   // The head kernel has stored the logits into pinned host memory; waiting for the stream
   // is the step's one synchronisation point (the reference's is the blocking cudaMemcpy in
   // tensor.cpp:65-68).  The returned CPU tensor is a view, valid until the next-but-one call.
-  FRHIP_CHECK(frhip_stream_sync(s));
-  {
-    // second step of the arg-max: greater value, then smaller index, over the per-slice pairs
-    const float *pairs = p.logits_host[cur] + p.n_logits;
-    float best = -INFINITY;
-    int32_t idx = p.n_logits;
-    for (int b = 0; b < DecodePlan::kArgmaxBlocks; b++) {
-      int32_t bi;
-      std::memcpy(&bi, pairs + 2 * b + 1, sizeof(bi));
-      if (pairs[2 * b] > best || (pairs[2 * b] == best && bi < idx)) {
-        best = pairs[2 * b];
-        idx = bi;
-      }
-    }
-    ex->last_argmax = idx < p.n_logits ? idx : 0;
-    ex->last_argmax_of = p.logits_host[cur];
-  }
+  FRHIP_CHECK(frhip_stream_sync(stream()));
+  settle(model, *ex, p, cur);
   if (p.owned_logits) {  // a tensor of the caller's own, as the reference returns (model.cpp:179-186)
     Tensor out = Tensor::Empty({p.n_logits}, DType::kFloat32, Device::kCPU);
     std::memcpy(out.data_ptr(), p.logits_host[cur], sizeof(float) * static_cast<size_t>(p.n_logits));
@@ -313,6 +379,74 @@ Tensor ModelForward(Model *model, Device device, int id) {
     return out;
   }
   return Tensor::FromPtr(p.logits_host[cur], {p.n_logits}, DType::kFloat32, Device::kCPU);
+}
+
+// `steps` greedy tokens starting from `first_id` with the host out of the loop: after the first token
+// (an ordinary ModelForward) every step's first kernel picks its token from the arg-max pairs of the step
+// before it, so the graphs are queued back to back and the host waits once per batch of at most
+// kChainIds - 1 steps instead of once per token (the top_k = 1 case of chat.cpp:56-92, where the host
+// sits between two forward passes).  The tokens, the logits of the last step and the state left behind
+// are those of the loop of ModelForward calls.  Returns false, having done nothing, when the fused
+// graph path is not the one in use; `last_logits`, if given, receives what the last Run would return.
+bool GreedyDecode(Model *model, int first_id, int steps, int *out_ids, Tensor *last_logits) {
+  const std::string &ver = model->version();
+  if (model->act_device() != Device::kHIP || std::getenv("FR_HIP_GENERIC") || std::getenv("FR_HIP_NO_GRAPH") ||
+      std::getenv("FR_HIP_GREEDY_ON_HOST") ||
+      !(ver == "4" || ver == "5" || ver == "5.1" || ver == "5.2"))
+    return false;
+  if (steps <= 0) return true;
+  Tensor lg = hip::ModelForward(model, Device::kHIP, first_id);
+  auto ex = extra_of(model);
+  DecodePlan &p = *ex->plan;
+  if (!p.use_graph) {  // the plan was made under FR_HIP_NO_GRAPH: finish token by token
+    out_ids[0] = ex->last_argmax;
+    for (int i = 1; i < steps; i++) {
+      lg = hip::ModelForward(model, Device::kHIP, out_ids[i - 1]);
+      out_ids[i] = ex->last_argmax;
+    }
+    if (last_logits) *last_logits = lg;
+    return true;
+  }
+  out_ids[0] = ex->last_argmax;
+  int done = 1;
+  while (done < steps) {
+    const int n = std::min(steps - done, DecodePlan::kChainIds - 1);
+    const uint32_t fed0 = p.fed;
+    int cur = p.parity;  // parity of the last token launched
+    int k = 0;
+    auto one = [&]() {
+      cur = p.parity;
+      launch_token(model, *ex, p, true);
+      k++;
+    };
+    if (p.chain_block_len >= 2) {
+      if (p.parity == 1 && k < n) one();
+      while (n - k >= p.chain_block_len) {
+        launch_chain_block(model, *ex, p);
+        cur = 1;
+        k += p.chain_block_len;
+      }
+    }
+    while (k < n) one();
+    FRHIP_CHECK(frhip_stream_sync(stream()));
+    // step done + k was fed the token out_ids[done + k - 1] and noted it in slot (fed0 + k)
+    for (int k = 1; k < n; k++) out_ids[done + k - 1] = p.chain_ids[(fed0 + k) % DecodePlan::kChainIds];
+    settle(model, *ex, p, cur);
+    out_ids[done + n - 1] = ex->last_argmax;
+    done += n;
+    if (last_logits) {
+      if (p.owned_logits) {
+        Tensor out = Tensor::Empty({p.n_logits}, DType::kFloat32, Device::kCPU);
+        std::memcpy(out.data_ptr(), p.logits_host[cur], sizeof(float) * static_cast<size_t>(p.n_logits));
+        ex->last_argmax_of = out.data_ptr();
+        lg = out;
+      } else {
+        lg = Tensor::FromPtr(p.logits_host[cur], {p.n_logits}, DType::kFloat32, Device::kCPU);
+      }
+    }
+  }
+  if (last_logits) *last_logits = lg;
+  return true;
 }
 
 // Index of the largest logit of the tensor `logits` if that tensor is the one the last one-token

@@ -148,6 +148,16 @@ int frhip_silu(const void *x, void *y, int dtype, size_t n, frhip_stream s);
 int frhip_embed_ring(const void *table, int n_rows, int row_bytes, const int32_t *ring, int ring_len,
                      uint32_t *counter_dev, void *out, frhip_stream s);
 
+/* Token feed of a greedy loop that the host does not take part in (the top_k = 1 case of
+ * chat.cpp:56-92, where the host picks the token between two forward passes): the token is the
+ * arg-max over `pairs`, the npairs {float value, int32 index} pairs frhip_argmax_blocks_f32 stored
+ * for the previous step's logits (device or pinned host memory; greater value, then smaller
+ * index; no finite maximum gives token 0).  It is stored to ids[*counter % ids_len] (device or
+ * pinned host memory) for the host to read after a later synchronisation, *counter advances,
+ * and that row of `table` is copied to `out`. */
+int frhip_embed_argmax(const void *table, int n_rows, int row_bytes, const void *pairs, int npairs, int32_t *ids,
+                       int ids_len, uint32_t *counter_dev, void *out, frhip_stream s);
+
 /* ---- fused one-token operators ------------------------------------------------ */
 /* Scratch the fused operators need: frhip_decode_workspace_bytes(C, F) bytes,
  * 256-byte aligned, owned by the caller, reusable across calls on one stream.

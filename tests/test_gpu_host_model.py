@@ -161,6 +161,55 @@ def test_kept_binary16_image_of_uint8_weights_gives_the_same_bits(spec, generic)
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("spec,strategy", [
+    ("v=4,L=4,C=512,F=2048,V=4096,seed=21", "hip fp16"),
+    ("v=4,L=4,C=512,F=2048,V=4096,seed=21", "hip int8"),
+    ("v=5.2,L=3,C=512,F=1792,V=4096,H=8,seed=22", "hip fp16"),
+    ("v=5,L=3,C=512,F=2048,V=4096,H=8,seed=23", "hip int8"),
+])
+def test_greedy_loop_kept_on_the_device_equals_the_loop_of_runs(spec, strategy):
+    """fr_greedy_decode on the fused path queues the steps back to back, each step's first kernel taking
+    its token from the arg-max pairs of the step before; FR_HIP_GREEDY_ON_HOST=1 is chat.cpp:56-92's
+    loop (Run, arg-max on the host, Run).  Same tokens, same logits afterwards, same state: bit for bit.
+    1 100 steps cross the 1 023-step batches the host waits for; a one-step and a two-step call and a
+    call right after a prompt in seq mode are covered too."""
+    prompt = [int(t) for t in np.random.default_rng(48).integers(0, 4096, 40)]
+
+    def run():
+        m = fr.Model("synthetic:" + spec, strategy)
+        out = []
+        for first, steps in ((7, 1), (8, 2), (9, 1100), (10, 33)):
+            ids, _ = m.greedy(first, steps)
+            out.append(ids.copy())
+        out.append(m.run(11).copy())
+        lg = m.run(prompt)
+        ids, _ = m.greedy(int(np.argmax(lg)), 50)
+        out.append(ids.copy())
+        out.append(m.run(12).copy())
+        out += [st for layer in m.states() for st in layer]
+        m.close()
+        return out
+
+    chained = run()
+    os.environ["FR_HIP_GREEDY_ON_HOST"] = "1"
+    try:
+        looped = run()
+    finally:
+        del os.environ["FR_HIP_GREEDY_ON_HOST"]
+    # the loop of runs, spelled out in Python, for the first calls
+    m = fr.Model("synthetic:" + spec, strategy)
+    for first, steps, got in ((7, 1, chained[0]), (8, 2, chained[1])):
+        t = first
+        for i in range(steps):
+            t = int(np.argmax(m.run(t)))
+            assert t == got[i]
+    m.close()
+    assert len(chained) == len(looped)
+    for a, b in zip(chained, looped):
+        assert np.array_equal(a, b)
+    assert len(set(chained[2].tolist())) > 1  # not a constant sequence
+
+
 def test_synthetic_model_and_cpp_greedy_loop():
     m = fr.Model("synthetic:v=4,L=2,C=256,F=1024,V=1024,seed=7", "hip int8")
     toks, secs = m.greedy(1, 16)
