@@ -276,28 +276,51 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chaine
                                       DecodePlan::kArgmaxBlocks, s));
 }
 
-// Replays (capturing it first, if need be) the graph of one token on the current parity and moves the
-// plan on to the next token; does not wait.
-static void launch_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chained) {
+// Captures `count` consecutive tokens, the first on parity `parity`, as one graph; nothing runs, and the
+// plan is left as it was.
+static frhip_graph capture_tokens(Model *model, ModelExtra &ex, DecodePlan &p, int parity, bool chained, int count) {
   frhip_stream s = stream();
+  const int saved = p.parity;
+  frhip_graph g = nullptr;
+  FRHIP_CHECK(frhip_graph_begin(s));
+  try {
+    p.parity = parity;
+    for (int k = 0; k < count; k++) {
+      issue_token(model, ex, p, chained);
+      p.parity = 1 - p.parity;
+    }
+  } catch (...) {
+    p.parity = saved;
+    frhip_graph_end(s, &g);
+    if (g) frhip_graph_destroy(g);
+    throw;
+  }
+  p.parity = saved;
+  FRHIP_CHECK(frhip_graph_end(s, &g));
+  return g;
+}
+
+// Every graph the plan can replay is captured the first time one of its kind is needed, both parities
+// at once, so that no later call pays for a capture because of the parity it happens to start on.
+static void ensure_graphs(Model *model, ModelExtra &ex, DecodePlan &p, bool chained) {
+  if (!p.use_graph) return;
+  for (int side = 0; side < 2; side++) {
+    frhip_graph &g = chained ? p.chain[side] : p.graph[side];
+    if (!g) g = capture_tokens(model, ex, p, side, chained, 1);
+  }
+  if (chained && p.chain_block_len >= 2 && !p.chain_block)
+    p.chain_block = capture_tokens(model, ex, p, 0, true, p.chain_block_len);
+}
+
+// Replays the graph of one token on the current parity and moves the plan on to the next token; does
+// not wait.
+static void launch_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chained) {
   const int cur = p.parity;
   if (!p.use_graph) {
     issue_token(model, ex, p, chained);
   } else {
-    frhip_graph &g = chained ? p.chain[cur] : p.graph[cur];
-    if (!g) {
-      FRHIP_CHECK(frhip_graph_begin(s));
-      try {
-        issue_token(model, ex, p, chained);
-      } catch (...) {
-        frhip_graph dead = nullptr;
-        frhip_graph_end(s, &dead);
-        if (dead) frhip_graph_destroy(dead);
-        throw;
-      }
-      FRHIP_CHECK(frhip_graph_end(s, &g));
-    }
-    FRHIP_CHECK(frhip_graph_launch(g, s));
+    ensure_graphs(model, ex, p, chained);
+    FRHIP_CHECK(frhip_graph_launch(chained ? p.chain[cur] : p.graph[cur], stream()));
   }
   p.fed++;  // the device counter advances when the first kernel of the step runs
   p.parity = 1 - cur;
@@ -306,25 +329,9 @@ static void launch_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chain
 // chain_block_len chained tokens in one graph (the gap between two graph launches on a stream is paid
 // once per block instead of once per token).  The plan must be on parity 0; it is again afterwards.
 static void launch_chain_block(Model *model, ModelExtra &ex, DecodePlan &p) {
-  frhip_stream s = stream();
   RV_CHECK(p.parity == 0 && p.chain_block_len % 2 == 0);
-  if (!p.chain_block) {
-    FRHIP_CHECK(frhip_graph_begin(s));
-    try {
-      for (int k = 0; k < p.chain_block_len; k++) {
-        issue_token(model, ex, p, true);
-        p.parity = 1 - p.parity;
-      }
-    } catch (...) {
-      p.parity = 0;
-      frhip_graph dead = nullptr;
-      frhip_graph_end(s, &dead);
-      if (dead) frhip_graph_destroy(dead);
-      throw;
-    }
-    FRHIP_CHECK(frhip_graph_end(s, &p.chain_block));
-  }
-  FRHIP_CHECK(frhip_graph_launch(p.chain_block, s));
+  ensure_graphs(model, ex, p, true);
+  FRHIP_CHECK(frhip_graph_launch(p.chain_block, stream()));
   p.fed += p.chain_block_len;
 }
 
