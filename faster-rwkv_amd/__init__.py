@@ -86,6 +86,7 @@ _SIGS = {
     "frhip_transpose": (_i, [_vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "frhip_silu": (_i, [_vp, _vp, _i, _sz, _vp]),
     "frhip_embed_ring": (_i, [_vp, _i, _i, _vp, _i, _vp, _vp, _vp]),
+    "frhip_embed_argmax": (_i, [_vp, _i, _i, _vp, _i, _vp, _i, _vp, _vp, _vp]),
     "frhip_decode_workspace_bytes": (_sz, [_i, _i]),
     "frhip_att_one_v4": (_i, [_i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 7),
     "frhip_ffn_one": (_i, [_i, _i] + [_vp] * 6 + [_WP] * 3 + [_vp, _vp, _i, _vp, _vp]),

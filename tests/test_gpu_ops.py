@@ -208,6 +208,56 @@ def test_argmax_blocks_first_of_ties(n, nblocks):
             assert vals[b] == -np.inf and idxs[b] == n
 
 
+def _host_rule(vals, idxs, n_rows):
+    """hip::ModelForward's second step of the arg-max (greater value, then smaller index; nothing
+    finite found: token 0)."""
+    best, at = -np.inf, n_rows
+    for v, i in zip(vals, idxs):
+        if v > best or (v == best and i < at):
+            best, at = v, int(i)
+    return at if at < n_rows else 0
+
+
+@pytest.mark.parametrize("case", ["random", "ties_across_slices", "all_minus_inf", "nan_slices", "nothing_found", "one_pair"])
+def test_embed_argmax_follows_the_host_rule(case):
+    """frhip_embed_argmax: the token picked from the per-slice pairs is the one the host's reduction
+    picks, it is noted in ids[counter % ids_len], the counter advances and the token's row is copied;
+    two calls in a row use two slots."""
+    n_rows, row = 1000, 256
+    tab = h(rng.standard_normal((n_rows, row)))
+    npairs = 1 if case == "one_pair" else 64
+    vals = rng.standard_normal(npairs).astype(np.float32)
+    idxs = rng.permutation(n_rows)[:npairs].astype(np.int32)
+    if case == "ties_across_slices":
+        vals[[5, 17, 40]] = 7.5
+    elif case == "all_minus_inf":
+        vals[:] = -np.inf
+    elif case == "nan_slices":
+        vals[::2] = np.nan
+    elif case == "nothing_found":  # what argmax_blocks reports for slices without a finite maximum
+        vals[:] = -np.inf
+        idxs[:] = n_rows
+    want = _host_rule(vals, idxs, n_rows)
+    if case == "ties_across_slices":
+        assert want == int(min(idxs[[5, 17, 40]]))
+    if case == "nothing_found":
+        assert want == 0
+    raw = np.empty(2 * npairs, np.float32)
+    raw[0::2] = vals
+    raw[1::2] = idxs.view(np.float32)
+    ids = DevBuf.empty(8, np.int32)
+    fr.check(L().frhip_fill(ids.ptr, fr.F32, 0.0, 8, None))
+    counter = keep(np.array([13], np.uint32))  # slot 13 % 8 = 5, then 6
+    out = DevBuf.empty(row, np.float16)
+    for call in range(2):
+        fr.check(L().frhip_embed_argmax(keep(tab).ptr, n_rows, 2 * row, keep(raw).ptr, npairs, ids.ptr, 8, counter.ptr,
+                                        out.ptr, None))
+        assert np.array_equal(out.numpy(), tab[want])
+        assert counter.numpy()[0] == 14 + call
+    got = ids.numpy()
+    assert got[5] == want and got[6] == want and not got[[0, 1, 2, 3, 4, 7]].any()
+
+
 def test_gather_rows():
     tab = h(rng.standard_normal((1000, 256)))
     ids = np.array([5, 999, 0, 5, 123], np.int32)
