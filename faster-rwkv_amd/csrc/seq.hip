@@ -201,10 +201,22 @@ struct Wkv4Seq {
 // before the recurrence touches the first, so a chunk of 16 steps costs one memory round trip
 // instead of 16 (with two waves per SIMD little else hides them: 8.3 -> 6.9 us and 10.7 -> 9.0 us
 // per launch at T = 1024).  What remains is launch, one round trip and the library expf (~28 VALU
-// instructions, six per token and channel over the three passes); a six-instruction exp2-based
-// exponential within 2 ulp brought the three passes from 28.4 to 25.2 us and was not kept: the
-// passes then no longer compute exactly what the one-token kernel does.
+// instructions; three per token and channel over the passes, one per pair: exp_pair below); a
+// six-instruction exp2-based exponential within 2 ulp was measured when the passes still took six
+// (28.4 -> 25.2 us) and was not kept: the passes then no longer compute exactly what the one-token
+// kernel does.
 constexpr int kScanB = 16;
+
+// p = max(a, b) (b on ties), ea = exp(a - p), eb = exp(b - p) with one exponential instead of two: the
+// argument of the other one is +0 and expf(+0) is exactly 1, so for finite a and b these are the bits
+// of the two calls.
+__device__ __forceinline__ void exp_pair(float a, float b, float& p, float& ea, float& eb) {
+  const bool first = a > b;
+  p = first ? a : b;
+  const float e = expf(first ? b - a : a - b);
+  ea = first ? 1.0f : e;
+  eb = first ? e : 1.0f;
+}
 
 __global__ __launch_bounds__(256) void wkv4_local_kernel(Wkv4Seq a) {
   const int c = blockIdx.x * 256 + threadIdx.x, ch = blockIdx.y;
@@ -224,9 +236,8 @@ __global__ __launch_bounds__(256) void wkv4_local_kernel(Wkv4Seq a) {
     for (int i = 0; i < kScanB; i++) {
       if (tb + i < t1) {
         const float k = kk[i], v = vv[i];
-        const float ww = w + pp;
-        const float p = (ww > k) ? ww : k;
-        const float e1 = expf(ww - p), e2 = expf(k - p);
+        float p, e1, e2;
+        exp_pair(w + pp, k, p, e1, e2);
         aa = e1 * aa + e2 * v;
         bb = e1 * bb + e2;
         pp = p;
@@ -268,9 +279,8 @@ __global__ __launch_bounds__(64) void wkv4_carry_kernel(Wkv4Seq a) {
         a.sp[o] = pp;
         const int len = min(a.Lc, a.T - ch * a.Lc);
         // the incoming state decays by len steps; the chunk's own tokens contribute its local state
-        const float pd = pp + (float)len * w;
-        const float p = (pd > lp[i]) ? pd : lp[i];
-        const float e1 = expf(pd - p), e2 = expf(lp[i] - p);
+        float p, e1, e2;
+        exp_pair(pp + (float)len * w, lp[i], p, e1, e2);
         aa = e1 * aa + e2 * la[i];
         bb = e1 * bb + e2 * lb[i];
         pp = p;
@@ -310,9 +320,8 @@ __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
 #pragma unroll
       for (int i = 0; i < PF; i++) {
         if (j0 + i < ch) {
-          const float pd = pp + pdw;
-          const float p = (pd > lp[i]) ? pd : lp[i];
-          const float e1 = expf(pd - p), e2 = expf(lp[i] - p);
+          float p, e1, e2;
+          exp_pair(pp + pdw, lp[i], p, e1, e2);
           aa = e1 * aa + e2 * la[i];
           bb = e1 * bb + e2 * lb[i];
           pp = p;
@@ -338,15 +347,11 @@ __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
       if (tb + i < t1) {
         const float k = kk[i], v = vv[i];
         // kernels/cuda/att.cu:43-60
-        float ww = u + k;
-        float p = (pp > ww) ? pp : ww;
-        float e1 = expf(pp - p), e2 = expf(ww - p);
+        float p, e1, e2;
+        exp_pair(pp, u + k, p, e1, e2);
         const float wkv = (e1 * aa + e2 * v) / (e1 * bb + e2);
         a.r[(size_t)(tb + i) * a.C + c] = rr[i] * (h1)wkv;
-        ww = w + pp;
-        p = (ww > k) ? ww : k;
-        e1 = expf(ww - p);
-        e2 = expf(k - p);
+        exp_pair(w + pp, k, p, e1, e2);
         aa = e1 * aa + e2 * v;
         bb = e1 * bb + e2;
         pp = p;
