@@ -4,6 +4,7 @@
 #pragma once
 
 #include <memory>
+#include <tuple>
 #include <vector>
 
 #include "frhip.h"
@@ -38,6 +39,12 @@ const frhip_weight *find_weight(const Tensor &t);
 // bytes per weight for as long as the model lives) instead of once per call into the
 // operator's workspace.  Both ways multiply by the same w^, so the results are the same bits.
 const frhip_weight *find_seq_weight(const Tensor &t, int rows);
+
+// ffn_seq with the halving that follows every sixth layer folded into its last epilogue (ops.cpp); same bits as
+// ffn_seq followed by scalar_div_(x, 2).
+std::tuple<Tensor, Tensor> ffn_seq_div2(const Tensor &x, const Tensor &sx, const Tensor &ln_w, const Tensor &ln_b,
+                                        const Tensor &k_mix, const Tensor &r_mix, const Tensor &kw, const Tensor &vw,
+                                        const Tensor &rw, bool div2);
 
 // Upload a host matrix in the reference's [K, N] layout and pack it for the kernels.
 // `dtype` kFloat16: src is binary16.  kInt8: src is binary16 and is quantised on the host

@@ -513,9 +513,10 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
       pi += 15;
     }
     const int off = ver[0] == '5' ? 2 : 4;
-    std::tie(x, st[off]) = ffn_seq(x, st[off], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5], p[pi + 6]);
+    // the halving after every sixth layer (model_forward_seq.cpp:163-165) rides in the ffn's last epilogue
+    std::tie(x, st[off]) = ffn_seq_div2(x, st[off], p[pi], p[pi + 1], p[pi + 2], p[pi + 3], p[pi + 4], p[pi + 5],
+                                        p[pi + 6], (i + 1) % 6 == 0);
     pi += 7;
-    if ((i + 1) % 6 == 0) scalar_div_(x, 2);
   }
   const frhip_weight *hw = find_seq_weight(p[pi + 2], full_output ? T : 1);
   RV_CHECK(hw != nullptr);

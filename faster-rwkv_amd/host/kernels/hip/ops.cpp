@@ -311,9 +311,11 @@ static Tensor seq_workspace(int T, int C, int F) {
 }
 
 // ffn_seq (reference: kernels/cuda/ffn_seq.cu:89-109).  x [T, C]; returns (x_out [T, C], LN(x)[T-1]).
-std::tuple<Tensor, Tensor> ffn_seq(const Tensor &x, const Tensor &sx, const Tensor &ln_w, const Tensor &ln_b,
-                                   const Tensor &k_mix, const Tensor &r_mix, const Tensor &kw, const Tensor &vw,
-                                   const Tensor &rw) {
+// `div2`: the result rows are halved in binary16 after the residual, as scalar_div_(x_out, 2) would
+// (model_forward_seq.cpp:163-165 does that as an operator of its own every sixth layer).
+std::tuple<Tensor, Tensor> ffn_seq_div2(const Tensor &x, const Tensor &sx, const Tensor &ln_w, const Tensor &ln_b,
+                                        const Tensor &k_mix, const Tensor &r_mix, const Tensor &kw, const Tensor &vw,
+                                        const Tensor &rw, bool div2) {
   RV_CHECK(x.dtype() == DType::kFloat16 && x.sizes().size() == 2);
   const int T = static_cast<int>(x.size(0)), C = static_cast<int>(x.size(1)), F = static_cast<int>(kw.size(1));
   frhip_weight d[3];
@@ -323,9 +325,15 @@ std::tuple<Tensor, Tensor> ffn_seq(const Tensor &x, const Tensor &sx, const Tens
   Tensor xx = Tensor::Empty({C}, x.dtype(), Device::kHIP);
   Tensor ws = seq_workspace(T, C, F);
   FRHIP_CHECK(frhip_ffn_seq(T, C, F, x.data_ptr(), sx.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), k_mix.data_ptr(),
-                            r_mix.data_ptr(), w[0], w[1], w[2], x_out.data_ptr(), xx.data_ptr(), 0, ws.data_ptr(),
-                            stream()));
+                            r_mix.data_ptr(), w[0], w[1], w[2], x_out.data_ptr(), xx.data_ptr(), div2 ? 1 : 0,
+                            ws.data_ptr(), stream()));
   return {x_out, xx};
+}
+
+std::tuple<Tensor, Tensor> ffn_seq(const Tensor &x, const Tensor &sx, const Tensor &ln_w, const Tensor &ln_b,
+                                   const Tensor &k_mix, const Tensor &r_mix, const Tensor &kw, const Tensor &vw,
+                                   const Tensor &rw) {
+  return ffn_seq_div2(x, sx, ln_w, ln_b, k_mix, r_mix, kw, vw, rw, false);
 }
 
 // att_seq, RWKV-4 (no counterpart upstream: kernels/default/model_forward_seq.cpp:111-112 throws).

@@ -134,6 +134,30 @@ def test_ffn_seq(T, C_, F_, quant):
     assert_close_f16(x_out.numpy(), ref_x, max_ulp=3, max_frac=0.2, what="x_out", floor_rms=1.0)
 
 
+@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (1024, 2048, 8192), (1, 512, 1024), (200, 768, 3072)])
+@pytest.mark.parametrize("quant", [False, True])
+def test_ffn_seq_with_the_halving_folded_in(T, C_, F_, quant):
+    """post_div2 = 1: the rows leave halved in binary16 after the residual, the bits of scalar_div_(x_out, 2) on
+    the result without it (model_forward_seq.cpp:163-165 halves the rows after every sixth layer); in the
+    launch split over K the halving sits in the reduction pass."""
+    g = np.random.default_rng(7000 + T)
+    x, sx = h(g.standard_normal((T, C_)) * 2), h(g.standard_normal(C_))
+    ln_w, ln_b = h(1 + 0.1 * g.standard_normal(C_)), h(0.1 * g.standard_normal(C_))
+    mk, mr = h(g.uniform(0, 1, C_)), h(g.uniform(0, 1, C_))
+    kw, _ = make_weight(h(g.standard_normal((C_, F_)) * 0.02), quant)
+    vw, _ = make_weight(h(g.standard_normal((F_, C_)) * 0.02), quant)
+    rw, _ = make_weight(h(g.standard_normal((C_, C_)) * 0.02), quant)
+    ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, F_))
+    outs = []
+    for div2 in (0, 1):
+        x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
+        fr.check(L().frhip_ffn_seq(T, C_, F_, keep(x).ptr, keep(sx).ptr, keep(ln_w).ptr, keep(ln_b).ptr, keep(mk).ptr,
+                                   keep(mr).ptr, kw.ref, vw.ref, rw.ref, x_out.ptr, xx_out.ptr, div2, ws.ptr, None))
+        outs.append((x_out.numpy(), xx_out.numpy()))
+    assert np.array_equal(outs[1][0], outs[0][0] / np.float16(2))
+    assert np.array_equal(outs[1][1], outs[0][1])  # the shift state is LN(x) of the last row: not halved
+
+
 def _state_v4(C_, fresh):
     if fresh:
         return np.zeros(C_, np.float32), np.zeros(C_, np.float32), np.full(C_, -1e30, np.float32)
