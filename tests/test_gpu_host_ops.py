@@ -176,6 +176,21 @@ def test_a_copy_of_states_is_a_snapshot_that_set_states_restores(tmp_path, versi
     m.restore(snap)
     third = [m.run(t) for t in (8, 9, 10, 11)]
     assert all(np.array_equal(a, b) for a, b in zip(first, third))
+    # the greedy loop kept on the device moves to fresh buffers as well while a snapshot is held
+    # (its graphs name the old ones), and gives the same tokens again from the restored state
+    m.restore(snap)
+    g1, _ = m.greedy(8, 37)
+    after1 = m.run(3).copy()
+    m.restore(snap)
+    g2, _ = m.greedy(8, 37)
+    after2 = m.run(3).copy()
+    assert np.array_equal(g1, g2) and np.array_equal(after1, after2)
+    m.restore(snap)
+    t, want = 8, []
+    for _ in range(37):
+        t = int(np.argmax(m.run(t)))
+        want.append(t)
+    assert want == g1.tolist()
     m.free_snapshot(snap)
     m.close()
 
