@@ -29,6 +29,7 @@ struct GemmSeg {
 struct GemmArgs {
   int M, K, nseg;
   int tile_start[kGemmMaxSeg + 1];  // first N-tile of each segment
+  size_t part_off[kGemmMaxSeg + 1]; // split launches: where each segment's [M][N] block starts within a slice of `partial` (floats); [nseg] = all
   // gemm_vw_kernel: a segment's tiles are vw_base (the first vw_wide of them vw_base + 1) blocks of 32 columns wide
   int vw_base[kGemmMaxSeg], vw_wide[kGemmMaxSeg], vw_maxw, vw_ns;
   GemmSeg seg[kGemmMaxSeg];
@@ -46,8 +47,12 @@ struct GemmArgs {
 // kDequantRows rows are expanded once to binary16 (the standalone dequantisation: the same bits as the
 // in-kernel one) and the launch takes the binary16 kernel.
 // partial: optional fp32 scratch of max_split slices of partial_stride floats (>= M * N each) for splitting K.
+// few_rows: optional fp32 scratch of few_rows_floats floats; with it a launch of so few rows that 64 x 128 tiles leave
+// at least half of the compute units idle goes out product by product, each split over K across the idle units.
+constexpr size_t kFewRowsFloats = (size_t)512 * 64 * 128;  // two 64 x 128 tiles per compute unit of a 256-unit part
+constexpr int kFewRowsMax = 256;                          // rows up to which the seq operators carry that scratch
 int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq = nullptr, float* partial = nullptr,
-                size_t partial_stride = 0, int max_split = 0);
+                size_t partial_stride = 0, int max_split = 0, float* few_rows = nullptr, size_t few_rows_floats = 0);
 constexpr int kDequantRows = FRHIP_SEQ_EXPAND_ROWS;
 // uint8 [N][K] -> binary16 [N][K] with the frozen formula (ops.hip)
 int dequant_u8_async(const unsigned char* q, const h1* mx, const h1* rx, const h1* my, const h1* ry, h1* dst, int K, int N,

@@ -517,7 +517,7 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
   }
   if (a.ksplit > 1) {
     GemmSeg sp = sg;  // this slice's sums go out as fp32; the epilogue proper follows in gemm_splitk_reduce_kernel
-    sp.out = a.partial + (size_t)blockIdx.z * a.partial_stride;
+    sp.out = a.partial + (size_t)blockIdx.z * a.partial_stride + a.part_off[sidx];
     sp.epi = G_STORE_F32;
     gemm_epilogue<BM>(a, sp, acc, m0, n0, M, N, lane, wm, wn);
   } else {
@@ -526,48 +526,99 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
 }
 
 // Adds the K slices of a split launch in slice order and applies the launch's epilogue; a thread
-// takes 8 consecutive outputs of a row (N % 8 == 0).
-__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a) {
-  const GemmSeg& sg = a.seg[0];
-  const size_t total = (size_t)a.M * sg.N;
-  const size_t o = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
-  if (o >= total) return;
-  float acc[8];
-  {
-    const f4v p0 = *reinterpret_cast<const f4v*>(a.partial + o), p1 = *reinterpret_cast<const f4v*>(a.partial + o + 4);
+// takes 16 consecutive outputs of a row (N % 16 == 0), the unit the batched sigmoid / silu work on.
+__global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(GemmArgs a) {
+  const size_t og = ((size_t)blockIdx.x * 64 + threadIdx.x) * 16;  // place within a slice, over all segments
+  if (og >= a.part_off[a.nseg]) return;
+  int sidx = 0;
 #pragma unroll
-    for (int i = 0; i < 4; i++) { acc[i] = p0[i]; acc[4 + i] = p1[i]; }
+  for (int i = 1; i < kGemmMaxSeg; i++) sidx += (i < a.nseg && og >= a.part_off[i]) ? 1 : 0;
+  const GemmSeg& sg = a.seg[sidx];
+  const size_t o = og - a.part_off[sidx];  // place within the segment's [M][N]
+  f16v acc;
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const f4v p = *reinterpret_cast<const f4v*>(a.partial + og + 4 * q);
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[4 * q + i] = p[i];
   }
-  for (int z = 1; z < a.ksplit; z++) {
-    const float* p = a.partial + (size_t)z * a.partial_stride + o;
-    const f4v p0 = *reinterpret_cast<const f4v*>(p), p1 = *reinterpret_cast<const f4v*>(p + 4);
+  // four slices are requested together and then added in slice order
+  for (int z0 = 1; z0 < a.ksplit; z0 += 4) {
+    f4v p[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) { acc[i] += p0[i]; acc[4 + i] += p1[i]; }
+    for (int j = 0; j < 4; j++) {
+      const int z = z0 + j < a.ksplit ? z0 + j : a.ksplit - 1;
+      const float* pz = a.partial + (size_t)z * a.partial_stride + og;
+#pragma unroll
+      for (int q = 0; q < 4; q++) p[j][q] = *reinterpret_cast<const f4v*>(pz + 4 * q);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (z0 + j < a.ksplit)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) acc[4 * q + i] += p[j][q][i];
   }
   if (sg.epi == G_STORE_F32) {
     float* out = static_cast<float*>(sg.out) + o;
 #pragma unroll
-    for (int i = 0; i < 8; i++) out[i] = acc[i];
+    for (int q = 0; q < 4; q++) {
+      f4v v;
+#pragma unroll
+      for (int i = 0; i < 4; i++) v[i] = acc[4 * q + i];
+      *reinterpret_cast<f4v*>(out + 4 * q) = v;
+    }
     return;
   }
-  h8 y;
-  if (sg.epi == G_STORE_F16) {
+  h1 y[16];
+  switch (sg.epi) {
+    case G_STORE_F16:
 #pragma unroll
-    for (int i = 0; i < 8; i++) y[i] = (h1)acc[i];
-  } else if (sg.epi == G_RESIDUAL) {
-    const h8 x = *reinterpret_cast<const h8*>(a.res_x + o);
+      for (int i = 0; i < 16; i++) y[i] = (h1)acc[i];
+      break;
+    case G_SIGMOID: sigmoid_h16(acc, y); break;
+    case G_SILU: silu_h16(acc, y); break;
+    case G_RELU2:
 #pragma unroll
-    for (int i = 0; i < 8; i++) y[i] = x[i] + (h1)acc[i];
-  } else {  // G_FFN_OUT
-    const h8 x = *reinterpret_cast<const h8*>(a.res_x + o), r = *reinterpret_cast<const h8*>(a.res_r + o);
+      for (int i = 0; i < 16; i++) {
+        const h1 t = (h1)acc[i];
+        y[i] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
+      }
+      break;
+    case G_RESIDUAL: {
+      const h8 x0 = *reinterpret_cast<const h8*>(a.res_x + o), x1 = *reinterpret_cast<const h8*>(a.res_x + o + 8);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      h1 v = __builtin_fmaf16((h1)acc[i], r[i], x[i]);
-      if (a.div2) v = v / (h1)2.0f;
-      y[i] = v;
+      for (int i = 0; i < 8; i++) {
+        y[i] = x0[i] + (h1)acc[i];
+        y[8 + i] = x1[i] + (h1)acc[8 + i];
+      }
+      break;
+    }
+    default: {  // G_FFN_OUT
+      const h8 x0 = *reinterpret_cast<const h8*>(a.res_x + o), x1 = *reinterpret_cast<const h8*>(a.res_x + o + 8);
+      const h8 r0 = *reinterpret_cast<const h8*>(a.res_r + o), r1 = *reinterpret_cast<const h8*>(a.res_r + o + 8);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        h1 v0 = __builtin_fmaf16((h1)acc[i], r0[i], x0[i]), v1 = __builtin_fmaf16((h1)acc[8 + i], r1[i], x1[i]);
+        if (a.div2) {
+          v0 = v0 / (h1)2.0f;
+          v1 = v1 / (h1)2.0f;
+        }
+        y[i] = v0;
+        y[8 + i] = v1;
+      }
+      break;
     }
   }
-  *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o) = y;
+  h8 lo, hi;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    lo[i] = y[i];
+    hi[i] = y[8 + i];
+  }
+  *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o) = lo;
+  *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o + 8) = hi;
 }
 
 template <int BM>
@@ -873,13 +924,14 @@ static int env_bk() {
 }
 
 int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq, float* partial, size_t partial_stride,
-                int max_split) {
+                int max_split, float* few_rows, size_t few_rows_floats) {
   if (a.M <= 0) return 0;
   if (a.K <= 0 || a.K % 64 != 0) return set_error(FRHIP_ESHAPE, "gemm: K must be a positive multiple of 64");
   if (u8 && dq && a.M >= kDequantRows) {
-    // Expanding N x K codes costs 3 bytes of traffic per weight; the uint8 kernel's in-flight dequantisation
-    // costs the launch about 0.4 x 2 T FLOP per weight at the binary16 kernel's rate: from a few hundred rows
-    // on, one expansion and the binary16 kernel win.
+    // Expanding N x K codes costs 3 bytes of traffic per weight.  The uint8 kernel's in-flight dequantisation costs a launch
+    // of many rows about 0.4 x 2 T FLOP per weight at the binary16 kernel's rate, and a launch of few rows cannot be spread
+    // over the idle compute units as the binary16 one can (few_rows below): with scratch for it, one expansion and the
+    // binary16 kernels win from a handful of rows on.
     h1* dst = static_cast<h1*>(dq);
     const unsigned char* qs[kGemmMaxSeg];
     const h1 *mxs[kGemmMaxSeg], *rxs[kGemmMaxSeg], *mys[kGemmMaxSeg], *rys[kGemmMaxSeg];
@@ -918,7 +970,54 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
   // second kernel adds the slices in order and applies the epilogue.  The sums are grouped by slice, so the result can
   // differ from the unsplit launch in the last fp32 bit before the rounding to binary16.  FRHIP_GEMM_SPLITK=0: off.
   static const bool splitk = !(getenv("FRHIP_GEMM_SPLITK") && atoi(getenv("FRHIP_GEMM_SPLITK")) == 0);
-  if (!u8 && ldw && splitk && !force_bm && partial && max_split >= 2 && a.nseg == 1 && a.K >= 4096 && a.seg[0].N % 8 == 0 &&
+  // Few rows (a short prompt): 64 x 128 tiles leave most compute units without a workgroup, and a workgroup pulls its
+  // weights through a ring of two K-steps (48 KB in flight), so a launch takes K / 64 round trips to memory however few
+  // rows there are (T = 64, 2048 x 2048: 16 workgroups, 17-25 us for 8 MB).  With scratch for the partial sums such a
+  // launch is split over K into as many slices as there are idle compute units (at least four K-steps each), and the
+  // reduction pass adds the slices in order and applies each product's epilogue.  A group that is too wide for that as a
+  // whole goes out product by product, so that its narrow members still can.  FRHIP_GEMM_FEW_ROWS=0: off.
+  static const bool few = !(getenv("FRHIP_GEMM_FEW_ROWS") && atoi(getenv("FRHIP_GEMM_FEW_ROWS")) == 0);
+  if (!u8 && ldw && splitk && few && !force_bm && few_rows) {
+    const int m64 = (a.M + 63) / 64, ksteps = a.K / kLdwBK, cus = compute_units();
+    bool eligible = (long)tiles * m64 * 2 <= cus && ksteps >= 4;
+    for (int sgi = 0; sgi < a.nseg; sgi++) eligible = eligible && a.seg[sgi].N % 16 == 0;
+    if (eligible) {
+      size_t cols = 0;
+      for (int sgi = 0; sgi < a.nseg; sgi++) {
+        a.part_off[sgi] = (size_t)a.M * cols;
+        cols += (size_t)a.seg[sgi].N;
+      }
+      a.part_off[a.nseg] = (size_t)a.M * cols;
+      const size_t stride = (a.part_off[a.nseg] + 63) / 64 * 64;
+      long S = cus / ((long)tiles * m64);
+      if (S > ksteps / 4) S = ksteps / 4;  // at least four K-steps per slice: twice the ring's depth in flight
+      if ((size_t)S * stride > few_rows_floats) S = (long)(few_rows_floats / stride);
+      if (S >= 2) {
+        a.ksplit = (int)S;
+        a.partial = few_rows;
+        a.partial_stride = stride;
+        gemm_ldw_launch<64>(dim3(tiles, m64, (unsigned)S), st, a);
+        if (int rc = check_launch(what)) return rc;
+        const size_t threads = (a.part_off[a.nseg] + 15) / 16;
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((threads + 63) / 64)), dim3(64), 0, st, a);
+        return check_launch(what);
+      }
+    } else if (a.nseg > 1 && ksteps >= 4) {
+      bool some = false;
+      for (int sgi = 0; sgi < a.nseg; sgi++)
+        some = some || ((long)((a.seg[sgi].N + BN - 1) / BN) * m64 * 2 <= cus && a.seg[sgi].N % 16 == 0);
+      if (some) {
+        for (int sgi = 0; sgi < a.nseg; sgi++) {
+          GemmArgs one = a;
+          one.nseg = 1;
+          one.seg[0] = a.seg[sgi];
+          if (int rc = launch_gemm(one, false, st, what, nullptr, nullptr, 0, 0, few_rows, few_rows_floats)) return rc;
+        }
+        return 0;
+      }
+    }
+  }
+  if (!u8 && ldw && splitk && !force_bm && partial && max_split >= 2 && a.nseg == 1 && a.K >= 4096 && a.seg[0].N % 16 == 0 &&
       (a.seg[0].epi == G_STORE_F16 || a.seg[0].epi == G_STORE_F32 || a.seg[0].epi == G_RESIDUAL || a.seg[0].epi == G_FFN_OUT) &&
       (size_t)a.M * a.seg[0].N <= partial_stride) {
     const long t128 = (long)tiles * m128;
@@ -929,10 +1028,12 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
       a.ksplit = S;
       a.partial = partial;
       a.partial_stride = partial_stride;
+      a.part_off[0] = 0;
+      a.part_off[1] = (size_t)a.M * a.seg[0].N;
       gemm_ldw_launch<128>(dim3(tiles, m128, S), st, a);
       if (int rc = check_launch(what)) return rc;
-      const size_t threads = ((size_t)a.M * a.seg[0].N + 7) / 8;
-      hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
+      const size_t threads = ((size_t)a.M * a.seg[0].N + 15) / 16;
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((threads + 63) / 64)), dim3(64), 0, st, a);
       return check_launch(what);
     }
   }
@@ -966,7 +1067,7 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
           GemmArgs one = a;
           one.nseg = 1;
           one.seg[0] = a.seg[sgi];
-          if (int rc = launch_gemm(one, false, st, what, nullptr, nullptr, 0, 0)) return rc;
+          if (int rc = launch_gemm(one, false, st, what, nullptr, nullptr, 0, 0, nullptr, 0)) return rc;
         }
         return 0;
       }

@@ -591,6 +591,8 @@ extern "C" size_t frhip_seq_workspace_bytes(int T, int C, int F) {
   const size_t tc = (size_t)T * C;
   // activations: 4 mixed inputs + g + gated (half), k v r y (fp32), vx [T][F] (half)
   size_t n = 6 * al256(2 * tc) + 4 * al256(4 * tc) + al256(2 * (size_t)T * F);
+  // short prompts: partial sums of the products split over K (launch_gemm's few_rows scratch)
+  if (T <= kFewRowsMax) n += al256(4 * kFewRowsFloats);
   // scan scratch: RWKV-4 6 x [nchunk][C] fp32 with nchunk <= T/8+1; RWKV-5 2 x [nchunk][C*64] fp32
   const size_t nchunk = (size_t)T / 8 + 1;
   n += 6 * al256(4 * nchunk * C) + 2 * al256(4 * nchunk * (size_t)C * 64);
@@ -603,6 +605,8 @@ namespace {
 struct SeqWs {
   h1 *m0, *m1, *m2, *m3, *g, *gated, *vx;
   float *f0, *f1, *f2, *f3;
+  float* few;        // kFewRowsFloats floats when T <= kFewRowsMax, else null
+  size_t few_floats;
   float* scan;
   h1* dq;  // binary16 expansion of one launch's uint8 weights
 };
@@ -620,6 +624,9 @@ SeqWs carve_seq(void* ws, int T, int C, int F) {
     *f = reinterpret_cast<float*>(p);
     p += al256(4 * tc);
   }
+  w.few = T <= kFewRowsMax ? reinterpret_cast<float*>(p) : nullptr;
+  w.few_floats = T <= kFewRowsMax ? kFewRowsFloats : 0;
+  if (w.few) p += al256(4 * kFewRowsFloats);
   w.vx = reinterpret_cast<h1*>(p);
   p += al256(2 * (size_t)T * F);
   w.scan = reinterpret_cast<float*>(p);
@@ -653,14 +660,14 @@ extern "C" int frhip_ffn_seq(int T, int C, int F, const void* x, const void* sx,
   gemm_add_seg(a, w.m1, rw, w.m2, G_SIGMOID);  // r
   gemm_add_seg(a, w.m0, kw, w.vx, G_RELU2);    // vx
   if (kw->dtype != rw->dtype) return set_error(FRHIP_EINVAL, "ffn_seq: key/receptance dtypes differ");
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "ffn_seq r,k", w.dq));
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "ffn_seq r,k", w.dq, nullptr, 0, 0, w.few, w.few_floats));
   GemmArgs b;
   memset(&b, 0, sizeof(b));
   b.M = T; b.K = F;
   b.res_x = (const h1*)x; b.res_r = w.m2; b.div2 = post_div2 ? 1 : 0;
   gemm_add_seg(b, w.vx, vw, x_out, G_FFN_OUT);
   // the four fp32 [T][C] buffers of the workspace (unused by ffn) take the partial sums of a K-split launch
-  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v", w.dq, w.f0, (size_t)(w.f1 - w.f0), 4);
+  return launch_gemm(b, vw->dtype == FRHIP_U8, st, "ffn_seq v", w.dq, w.f0, (size_t)(w.f1 - w.f0), 4, w.few, w.few_floats);
 }
 
 // RWKV-4 sequence attention.  The reference has no such operator
@@ -693,7 +700,7 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   gemm_add_seg(a, w.m0, kw, w.f0, G_STORE_F32);  // k
   gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
   gemm_add_seg(a, w.m2, rw, w.m3, G_SIGMOID);    // r
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v4 k,v,r", w.dq));
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v4 k,v,r", w.dq, nullptr, 0, 0, w.few, w.few_floats));
 
   Wkv4Seq q;
   q.T = T; q.C = C;
@@ -724,7 +731,7 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   b.M = T; b.K = C;
   b.res_x = (const h1*)x;
   gemm_add_seg(b, w.m3, ow, x_out, G_RESIDUAL);
-  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v4 out", w.dq);
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v4 out", w.dq, nullptr, 0, 0, w.few, w.few_floats);
 }
 
 // Shared by RWKV-5.0 (no gate, u and w per head) and RWKV-5.2.
@@ -759,7 +766,7 @@ static int att_seq_v5_impl(bool v50, int T, int C, int H, const void* x, const v
   gemm_add_seg(a, w.m1, vw, w.f1, G_STORE_F32);  // v
   gemm_add_seg(a, w.m2, rw, w.f2, G_STORE_F32);  // r
   if (!v50) gemm_add_seg(a, w.m3, gw, w.g, G_SILU);  // g
-  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5 k,v,r,g", w.dq));
+  FR_TRY(launch_gemm(a, kw->dtype == FRHIP_U8, st, "att_seq_v5 k,v,r,g", w.dq, nullptr, 0, 0, w.few, w.few_floats));
 
   Wkv5Seq q;
   q.T = T; q.C = C; q.H = H;
@@ -782,7 +789,7 @@ static int att_seq_v5_impl(bool v50, int T, int C, int H, const void* x, const v
   b.M = T; b.K = C;
   b.res_x = (const h1*)x;
   gemm_add_seg(b, w.gated, ow, x_out, G_RESIDUAL);
-  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5 out", w.dq);
+  return launch_gemm(b, ow->dtype == FRHIP_U8, st, "att_seq_v5 out", w.dq, nullptr, 0, 0, w.few, w.few_floats);
 }
 
 // att_seq_v5_2 (kernels/cuda/att_seq.cu:368-423,464-493).

@@ -100,11 +100,12 @@ int frhip_pack_transpose(const void *src_kn, void *dst_nk, int K, int N, int ele
  * frhip_gemm multiplies by exactly this w^; the one-token operators (frhip_gemv, att, ffn,
  * head) evaluate the same formula in fp32 without the final rounding of w^. */
 int frhip_dequant_u8(const frhip_weight *w, void *dst_nk_f16, frhip_stream s);
-/* From this many rows on, frhip_gemm and the *_seq operators multiply uint8 weights by expanding
- * them to binary16 first (into their workspace, once per call).  A caller with memory to spare can
+/* From this many rows on, the *_seq operators multiply uint8 weights by expanding them to binary16
+ * first (into their workspace, once per call; below, and in frhip_gemm, which has no workspace,
+ * the codes are dequantised on their way into the product).  A caller with memory to spare can
  * keep the frhip_dequant_u8 image of a weight and pass it as an FRHIP_F16 weight for such calls:
  * the products see the same w^ and the results are the same bits. */
-#define FRHIP_SEQ_EXPAND_ROWS 192
+#define FRHIP_SEQ_EXPAND_ROWS 4
 
 /* ---- primitive operators (names of kernels/kernels.h) ------------------------ */
 /* layernorm: kernels/cuda/layer_norm.cu:101-130.  dtype FRHIP_F16 or FRHIP_F32 for x, gamma, beta, y. */

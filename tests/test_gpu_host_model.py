@@ -131,8 +131,8 @@ def test_seq_mode_equals_one_token_steps_and_oracle(model_files, strategy):
 def test_kept_binary16_image_of_uint8_weights_gives_the_same_bits(spec, generic):
     """FR_HIP_SEQ_IMAGE=1: prompts of FRHIP_SEQ_EXPAND_ROWS rows or more multiply the kept binary16
     image of the uint8 weights instead of one expanded per call; w^ is the same, so logits (last
-    row and every row) and the state left behind are the same bits.  Shorter prompts and one-token
-    steps still read the codes."""
+    row and every row) and the state left behind are the same bits.  One-token steps still read the
+    codes."""
     ids = [int(t) for t in np.random.default_rng(47).integers(0, 2048, 300)]
 
     def run():
