@@ -115,7 +115,11 @@ def _common(C_):
 
 # (1024, 2048, 8192): r and k as separate one-round launches, the value product split over K in two slices;
 # (300, 2048, 8192): the value product in four slices over ragged row tiles; (512, 2560, 8960): three slices of 47, 47 and 46 K-steps
-@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1024, 2048, 8192), (512, 2560, 8960), (1, 512, 1024), (33, 768, 3072), (3000, 512, 1792)])
+# (16, 2048, 8192), (130, 2048, 8192), (200, 2560, 8960): short prompts at full width -- products split over K across the idle compute
+# units: r,k grouped in one split launch (16 rows), product by product because the group is too wide (130, 200 rows), the value
+# product in 16 and in fewer slices
+@pytest.mark.parametrize("T,C_,F_", [(64, 512, 1792), (300, 2048, 8192), (1024, 2048, 8192), (512, 2560, 8960), (1, 512, 1024), (33, 768, 3072), (3000, 512, 1792),
+                                     (16, 2048, 8192), (130, 2048, 8192), (200, 2560, 8960)])
 @pytest.mark.parametrize("quant", [False, True])
 def test_ffn_seq(T, C_, F_, quant):
     g = np.random.default_rng(5000 + T) if T >= 512 else rng  # the full-size cases draw from a stream of their own
@@ -165,7 +169,7 @@ def _state_v4(C_, fresh):
             rng.standard_normal(C_).astype(np.float32))
 
 
-@pytest.mark.parametrize("T,C_", [(64, 512), (1024, 2048), (1, 512), (37, 768), (3000, 512)])  # 3000: a long, ragged prompt (94 chunks)
+@pytest.mark.parametrize("T,C_", [(64, 512), (1024, 2048), (1, 512), (37, 768), (3000, 512), (24, 2048), (150, 2048)])  # 3000: a long, ragged prompt (94 chunks); 24, 150: short prompts at full width (split products)
 @pytest.mark.parametrize("quant", [False, True])
 @pytest.mark.parametrize("fresh", [True, False])
 def test_att_seq_v4(T, C_, quant, fresh):
@@ -197,7 +201,7 @@ def test_att_seq_v4(T, C_, quant, fresh):
     assert np.abs(po_.numpy() - ref[4]).max() < 30  # offsets stay in a sane range
 
 
-@pytest.mark.parametrize("T,C_,H_", [(48, 512, 8), (512, 2560, 40), (1, 512, 8), (77, 512, 8), (3000, 512, 8)])
+@pytest.mark.parametrize("T,C_,H_", [(48, 512, 8), (512, 2560, 40), (1, 512, 8), (77, 512, 8), (3000, 512, 8), (40, 2560, 40)])  # (40, 2560, 40): k,v,r,g of a short prompt in one split launch
 @pytest.mark.parametrize("quant", [False, True])
 def test_att_seq_v5_2(T, C_, H_, quant):
     S_ = C_ // H_
