@@ -525,45 +525,54 @@ __global__ __launch_bounds__(kLdwThreads) void gemm_ldw_kernel(GemmArgs a) {
   }
 }
 
-// Adds the K slices of a split launch in slice order and applies the launch's epilogue; a thread
-// takes 16 consecutive outputs of a row (N % 16 == 0), the unit the batched sigmoid / silu work on.
-__global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(GemmArgs a) {
-  const size_t og = ((size_t)blockIdx.x * 64 + threadIdx.x) * 16;  // place within a slice, over all segments
-  if (og >= a.part_off[a.nseg]) return;
-  int sidx = 0;
+// Adds the K slices of a split launch in slice order and applies each product's epilogue; a thread
+// takes W consecutive outputs of a row: 16, the unit the batched sigmoid / silu work on, when one of
+// the epilogues is one of those, else 8 (N % 16 == 0 either way).
+// og: the thread's place within a slice, over all segments; o: within its segment's [M][N]
+template <int W>
+__device__ __forceinline__ void splitk_reduce_body(const GemmArgs& a, const GemmSeg& sg, size_t og, size_t o) {
+  constexpr int Q = W / 4;
+  float acc[W];
 #pragma unroll
-  for (int i = 1; i < kGemmMaxSeg; i++) sidx += (i < a.nseg && og >= a.part_off[i]) ? 1 : 0;
-  const GemmSeg& sg = a.seg[sidx];
-  const size_t o = og - a.part_off[sidx];  // place within the segment's [M][N]
-  f16v acc;
-#pragma unroll
-  for (int q = 0; q < 4; q++) {
+  for (int q = 0; q < Q; q++) {
     const f4v p = *reinterpret_cast<const f4v*>(a.partial + og + 4 * q);
 #pragma unroll
     for (int i = 0; i < 4; i++) acc[4 * q + i] = p[i];
   }
-  // four slices are requested together and then added in slice order
-  for (int z0 = 1; z0 < a.ksplit; z0 += 4) {
-    f4v p[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int z = z0 + j < a.ksplit ? z0 + j : a.ksplit - 1;
+  // many slices (a short prompt's launch): four are requested together and then added in slice order
+  if (a.ksplit <= 4) {
+    for (int z = 1; z < a.ksplit; z++) {
       const float* pz = a.partial + (size_t)z * a.partial_stride + og;
 #pragma unroll
-      for (int q = 0; q < 4; q++) p[j][q] = *reinterpret_cast<const f4v*>(pz + 4 * q);
+      for (int q = 0; q < Q; q++) {
+        const f4v p = *reinterpret_cast<const f4v*>(pz + 4 * q);
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[4 * q + i] += p[i];
+      }
+    }
+  } else
+  for (int z0 = 1; z0 < a.ksplit; z0 += 4) {
+    f4v p[4][Q];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      if (z0 + j < a.ksplit) {
+        const float* pz = a.partial + (size_t)(z0 + j) * a.partial_stride + og;
+#pragma unroll
+        for (int q = 0; q < Q; q++) p[j][q] = *reinterpret_cast<const f4v*>(pz + 4 * q);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; j++)
       if (z0 + j < a.ksplit)
 #pragma unroll
-        for (int q = 0; q < 4; q++)
+        for (int q = 0; q < Q; q++)
 #pragma unroll
           for (int i = 0; i < 4; i++) acc[4 * q + i] += p[j][q][i];
   }
   if (sg.epi == G_STORE_F32) {
     float* out = static_cast<float*>(sg.out) + o;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
+    for (int q = 0; q < Q; q++) {
       f4v v;
 #pragma unroll
       for (int i = 0; i < 4; i++) v[i] = acc[4 * q + i];
@@ -571,54 +580,83 @@ __global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(GemmArgs a) {
     }
     return;
   }
-  h1 y[16];
+  h1 y[W];
   switch (sg.epi) {
     case G_STORE_F16:
 #pragma unroll
-      for (int i = 0; i < 16; i++) y[i] = (h1)acc[i];
+      for (int i = 0; i < W; i++) y[i] = (h1)acc[i];
       break;
-    case G_SIGMOID: sigmoid_h16(acc, y); break;
-    case G_SILU: silu_h16(acc, y); break;
+    case G_SIGMOID:
+    case G_SILU:
+      if constexpr (W == 16) {
+        f16v c;
+#pragma unroll
+        for (int i = 0; i < 16; i++) c[i] = acc[i];
+        if (sg.epi == G_SIGMOID) sigmoid_h16(c, y); else silu_h16(c, y);
+      }
+      break;
     case G_RELU2:
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
+      for (int i = 0; i < W; i++) {
         const h1 t = (h1)acc[i];
         y[i] = (t > (h1)0.0f) ? (t * t) : (h1)0.0f;
       }
       break;
-    case G_RESIDUAL: {
-      const h8 x0 = *reinterpret_cast<const h8*>(a.res_x + o), x1 = *reinterpret_cast<const h8*>(a.res_x + o + 8);
+    case G_RESIDUAL:
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        y[i] = x0[i] + (h1)acc[i];
-        y[8 + i] = x1[i] + (h1)acc[8 + i];
+      for (int g = 0; g < W / 8; g++) {
+        const h8 x = *reinterpret_cast<const h8*>(a.res_x + o + 8 * g);
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[8 * g + i] = x[i] + (h1)acc[8 * g + i];
       }
       break;
-    }
-    default: {  // G_FFN_OUT
-      const h8 x0 = *reinterpret_cast<const h8*>(a.res_x + o), x1 = *reinterpret_cast<const h8*>(a.res_x + o + 8);
-      const h8 r0 = *reinterpret_cast<const h8*>(a.res_r + o), r1 = *reinterpret_cast<const h8*>(a.res_r + o + 8);
+    default:  // G_FFN_OUT
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        h1 v0 = __builtin_fmaf16((h1)acc[i], r0[i], x0[i]), v1 = __builtin_fmaf16((h1)acc[8 + i], r1[i], x1[i]);
-        if (a.div2) {
-          v0 = v0 / (h1)2.0f;
-          v1 = v1 / (h1)2.0f;
+      for (int g = 0; g < W / 8; g++) {
+        const h8 x = *reinterpret_cast<const h8*>(a.res_x + o + 8 * g), r = *reinterpret_cast<const h8*>(a.res_r + o + 8 * g);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          h1 v = __builtin_fmaf16((h1)acc[8 * g + i], r[i], x[i]);
+          if (a.div2) v = v / (h1)2.0f;
+          y[8 * g + i] = v;
         }
-        y[i] = v0;
-        y[8 + i] = v1;
       }
       break;
-    }
   }
-  h8 lo, hi;
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    lo[i] = y[i];
-    hi[i] = y[8 + i];
+  for (int g = 0; g < W / 8; g++) {
+    h8 v;
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = y[8 * g + i];
+    *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o + 8 * g) = v;
   }
-  *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o) = lo;
-  *reinterpret_cast<h8*>(static_cast<h1*>(sg.out) + o + 8) = hi;
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a) {
+  const size_t og = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * W;
+  if (a.nseg == 1) {  // the segment's description stays in scalar registers
+    if (og < a.part_off[1]) splitk_reduce_body<W>(a, a.seg[0], og, og);
+    return;
+  }
+  if (og >= a.part_off[a.nseg]) return;
+  int sidx = 0;
+#pragma unroll
+  for (int i = 1; i < kGemmMaxSeg; i++) sidx += (i < a.nseg && og >= a.part_off[i]) ? 1 : 0;
+  splitk_reduce_body<W>(a, a.seg[sidx], og, og - a.part_off[sidx]);
+}
+
+// Small reductions go out in workgroups of one wave, so that they spread over the compute units.
+static void launch_splitk_reduce(hipStream_t st, const GemmArgs& a) {
+  bool wide = false;
+  for (int i = 0; i < a.nseg; i++) wide = wide || a.seg[i].epi == G_SIGMOID || a.seg[i].epi == G_SILU;
+  const size_t threads = (a.part_off[a.nseg] + (wide ? 15 : 7)) / (wide ? 16 : 8);
+  const unsigned block = threads >= 65536 ? 256 : 64;
+  const dim3 grid((unsigned)((threads + block - 1) / block));
+  if (wide)
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<16>, grid, dim3(block), 0, st, a);
+  else
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<8>, grid, dim3(block), 0, st, a);
 }
 
 template <int BM>
@@ -998,8 +1036,7 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
         a.partial_stride = stride;
         gemm_ldw_launch<64>(dim3(tiles, m64, (unsigned)S), st, a);
         if (int rc = check_launch(what)) return rc;
-        const size_t threads = (a.part_off[a.nseg] + 15) / 16;
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((threads + 63) / 64)), dim3(64), 0, st, a);
+        launch_splitk_reduce(st, a);
         return check_launch(what);
       }
     } else if (a.nseg > 1 && ksteps >= 4) {
@@ -1032,8 +1069,7 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
       a.part_off[1] = (size_t)a.M * a.seg[0].N;
       gemm_ldw_launch<128>(dim3(tiles, m128, S), st, a);
       if (int rc = check_launch(what)) return rc;
-      const size_t threads = ((size_t)a.M * a.seg[0].N + 15) / 16;
-      hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((threads + 63) / 64)), dim3(64), 0, st, a);
+      launch_splitk_reduce(st, a);
       return check_launch(what);
     }
   }
