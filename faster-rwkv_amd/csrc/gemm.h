@@ -50,7 +50,7 @@ struct GemmArgs {
 // few_rows: optional fp32 scratch of few_rows_floats floats; with it a launch of so few rows that 64 x 128 tiles leave
 // at least half of the compute units idle goes out product by product, each split over K across the idle units.
 constexpr size_t kFewRowsFloats = (size_t)512 * 64 * 128;  // two 64 x 128 tiles per compute unit of a 256-unit part
-constexpr int kFewRowsMax = 256;                          // rows up to which the seq operators carry that scratch
+constexpr int kFewRowsMax = 360;                          // rows up to which the seq operators carry that scratch
 int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq = nullptr, float* partial = nullptr,
                 size_t partial_stride = 0, int max_split = 0, float* few_rows = nullptr, size_t few_rows_floats = 0);
 constexpr int kDequantRows = FRHIP_SEQ_EXPAND_ROWS;
