@@ -479,7 +479,7 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
   if (std::getenv("FR_HIP_GENERIC")) return def::ModelForwardSeq(model, device, ids, full_output);
   RV_CHECK(!ids.empty());
   // A prompt of two or three tokens is quicker as one-token steps (0.7 ms each for the 1.5B shape) than as a pass
-  // of the seq operators, which for so few rows costs its ~270 launches (1.9 ms); FR_HIP_SEQ_ALWAYS=1: never.
+  // of the seq operators, which for so few rows costs its ~290 launches (1.9 ms); FR_HIP_SEQ_ALWAYS=1: never.
   if (!full_output && ids.size() < 4 && !std::getenv("FR_HIP_SEQ_ALWAYS")) {
     Tensor out;
     for (int id : ids) out = hip::ModelForward(model, device, id);
