@@ -202,15 +202,19 @@ def rwkv5_extra(fr):
     m = fr.Model("synthetic:v=5.2,L=32,C=2560,F=8960,V=65536,H=40,seed=1238", "hip int8")
     ids = np.random.default_rng(44).integers(0, V_, 512)
     best = 1e9
-    for _ in range(3):
-        m.reset()
-        t0 = time.perf_counter()
-        lg = m.run(ids)
-        best = min(best, time.perf_counter() - t0)
+    os.environ["FR_HIP_SEQ_IMAGE"] = "0"  # the uint8 weights expanded to binary16 per call, nothing kept
+    try:
+        for _ in range(3):
+            m.reset()
+            t0 = time.perf_counter()
+            lg = m.run(ids)
+            best = min(best, time.perf_counter() - t0)
+    finally:
+        del os.environ["FR_HIP_SEQ_IMAGE"]
     m.greedy(int(np.argmax(lg)), 16)
     _, secs = m.greedy(17, 256)
-    # the same prompt with the binary16 image of the uint8 weights kept on the device (FR_HIP_SEQ_IMAGE=1:
-    # 2 more bytes per weight, no expansion per call); the first pass makes the images and is not timed
+    # the same prompt with the binary16 image of the uint8 weights kept on the device (FR_HIP_SEQ_IMAGE=1, the default
+    # on a device of this size: 2 more bytes per weight, no expansion per call); the first pass makes the images and is not timed
     os.environ["FR_HIP_SEQ_IMAGE"] = "1"
     try:
         kept = 1e9
@@ -225,8 +229,8 @@ def rwkv5_extra(fr):
     assert np.array_equal(lg, lg2), "kept binary16 image changed the logits"
     m.close()
     wbytes = 32 * 85196800 + 167772160  # uint8 codes of every matrix, once per token
-    return {"rwkv5_3b_int8_prefill_T512_ms": round(best * 1e3, 2), "rwkv5_3b_int8_prefill_tok_s": round(512 / best, 1),
-            "rwkv5_3b_int8_prefill_T512_kept_image_ms": round(kept * 1e3, 2),
+    return {"rwkv5_3b_int8_prefill_T512_ms": round(kept * 1e3, 2), "rwkv5_3b_int8_prefill_tok_s": round(512 / kept, 1),
+            "rwkv5_3b_int8_prefill_T512_expanded_per_call_ms": round(best * 1e3, 2),
             "rwkv5_3b_int8_decode_tok_s": round(256 / secs, 1),
             "rwkv5_3b_int8_decode_weight_GBs": round(wbytes * 256 / secs / 1e9, 1)}
 

@@ -27,6 +27,7 @@ struct PackedWeight {
   // (frhip_dequant_u8) and its description.  Freed with the weight.
   Tensor image;
   frhip_weight image_desc{};
+  bool no_image = false;  // the image could not be allocated once: not tried again
 };
 
 void register_weight(const void *data_ptr, std::shared_ptr<PackedWeight> w);
@@ -34,10 +35,11 @@ void unregister_weight(const void *data_ptr);
 // nullptr when `t` is not a packed weight.
 const frhip_weight *find_weight(const Tensor &t);
 // The description to hand to a product over `rows` rows of activations.  The same as
-// find_weight unless FR_HIP_SEQ_IMAGE=1 is set, the weight is uint8 and rows >=
-// FRHIP_SEQ_EXPAND_ROWS: then the weight's binary16 image, expanded once and kept (2 more
-// bytes per weight for as long as the model lives) instead of once per call into the
-// operator's workspace.  Both ways multiply by the same w^, so the results are the same bits.
+// find_weight unless images are kept (FR_HIP_SEQ_IMAGE=1, or unset on a device with 128 GB
+// or more; =0: never), the weight is uint8 and rows >= FRHIP_SEQ_EXPAND_ROWS: then the
+// weight's binary16 image, expanded once and kept (2 more bytes per weight for as long as
+// the model lives) instead of once per call into the operator's workspace.  Both ways
+// multiply by the same w^, so the results are the same bits.
 const frhip_weight *find_seq_weight(const Tensor &t, int rows);
 
 // ffn_seq with the halving that follows every sixth layer folded into its last epilogue (ops.cpp); same bits as

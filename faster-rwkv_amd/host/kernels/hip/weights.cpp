@@ -51,20 +51,39 @@ const frhip_weight *find_weight(const Tensor &t) {
   return it == table().end() ? nullptr : &it->second->desc;
 }
 
+// FR_HIP_SEQ_IMAGE=1 / 0 decides (read per call, like FR_HIP_GENERIC); unset: kept on a device with 128 GB or more,
+// where the image of even a 14B model (28 GB beside 14 GB of codes) is a small part of the memory.
+static bool keep_images() {
+  if (const char *e = std::getenv("FR_HIP_SEQ_IMAGE")) return std::atoi(e) != 0;
+  static const bool roomy = [] {
+    (void)stream();  // the device is initialised
+    char name[128];
+    int cus = 0;
+    size_t total = 0;
+    if (frhip_device_info(name, sizeof(name), &cus, &total) != 0) return false;
+    return total >= (static_cast<size_t>(128) << 30);
+  }();
+  return roomy;
+}
+
 const frhip_weight *find_seq_weight(const Tensor &t, int rows) {
-  const char *e = std::getenv("FR_HIP_SEQ_IMAGE");  // read per call, like FR_HIP_GENERIC
-  const bool keep = e && std::atoi(e) != 0;
-  if (!keep || rows < FRHIP_SEQ_EXPAND_ROWS) return find_weight(t);
+  if (rows < FRHIP_SEQ_EXPAND_ROWS || !keep_images()) return find_weight(t);
   if (!t.defined() || t.device() != Device::kHIP) return nullptr;
   std::lock_guard<std::mutex> lock(g_mu);
   auto it = table().find(t.data_ptr());
   if (it == table().end()) return nullptr;
   PackedWeight &w = *it->second;
-  if (w.desc.dtype != FRHIP_U8) return &w.desc;
+  if (w.desc.dtype != FRHIP_U8 || w.no_image) return &w.desc;
   if (!w.image.defined()) {
+    Tensor img;
+    try {
+      img = Tensor::Empty({static_cast<LengthType>(w.desc.N), static_cast<LengthType>(w.desc.K)}, DType::kFloat16,
+                          Device::kHIP);
+    } catch (const std::exception &) {  // no room: this weight is expanded per call, as without images
+      w.no_image = true;
+      return &w.desc;
+    }
     // on the backend's stream, like every product that will read it
-    Tensor img = Tensor::Empty({static_cast<LengthType>(w.desc.N), static_cast<LengthType>(w.desc.K)}, DType::kFloat16,
-                               Device::kHIP);
     FRHIP_CHECK(frhip_dequant_u8(&w.desc, img.data_ptr(), stream()));
     w.image = img;
     w.image_desc = frhip_weight{};
