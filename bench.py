@@ -171,6 +171,21 @@ def probe_bandwidth(fr, nbytes=2 << 30, reps=5):
     return out
 
 
+def prompt_only(fr, T):
+    """One prompt length alone (profiling aid): best of 4 passes over T tokens of the fp16 model."""
+    cfg = CONFIGS["fp16"]
+    m = fr.Model(cfg["spec"], cfg["strategy"])
+    ids = np.random.default_rng(43).integers(0, V_, T)
+    best = 1e9
+    for _ in range(4):
+        m.reset()
+        t0 = time.perf_counter()
+        m.run(ids)
+        best = min(best, time.perf_counter() - t0)
+    m.close()
+    return {"prompt_len": T, "prompt_ms": round(best * 1e3, 3), "prompt_tok_s": round(T / best, 1)}
+
+
 def prefill_extra(fr):
     """BASELINE configuration 4: T=1024 seq-mode prefill of the same fp16 model."""
     cfg = CONFIGS["fp16"]
@@ -417,6 +432,8 @@ def main():
                     help="only time the prompt pass's products standalone, beside torch.matmul on the same shapes, and print that")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run the T=1024 seq-mode prefill side measurement and print it (profiling aid)")
+    ap.add_argument("--prompt-len", type=int, default=0,
+                    help="only run a prompt of this many tokens through the fp16 model and print its time (profiling aid)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs batch-1 decode on ONE GPU; --gpus %d is not supported "
@@ -433,6 +450,9 @@ def main():
         return
     if args.gemm_probe:
         print(json.dumps(probe_gemm(fr)), flush=True)
+        return
+    if args.prompt_len > 0:
+        print(json.dumps(prompt_only(fr, args.prompt_len)), flush=True)
         return
     if args.prefill_only:
         print(json.dumps(prefill_extra(fr)), flush=True)
