@@ -1039,7 +1039,7 @@ int launch_gemm(GemmArgs& a, bool u8, hipStream_t st, const char* what, void* dq
         launch_splitk_reduce(st, a);
         return check_launch(what);
       }
-    } else if (a.nseg > 1 && ksteps >= 4) {
+    } else if (a.nseg > 1 && ksteps >= 4 && (long)tiles * m64 < cus) {  // a group that fills the part as it is stays one launch
       bool some = false;
       for (int sgi = 0; sgi < a.nseg; sgi++)
         some = some || ((long)((a.seg[sgi].N + BN - 1) / BN) * m64 * 2 <= cus && a.seg[sgi].N % 16 == 0);
