@@ -378,7 +378,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
 // needs scalar instructions only.  `lds` is the destination's LDS byte address (lane l writes 16 bytes
 // at lds + 16 l); the wait counts are the caller's business, as with the builtin.
 __device__ __forceinline__ void load_lds_saddr(unsigned voff, const void* sbase, unsigned lds) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
 }
 
 // The same address for every lane, in scalar registers (the compiler cannot always prove it).

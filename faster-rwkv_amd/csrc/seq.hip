@@ -191,9 +191,9 @@ struct Wkv4Seq {
   int T, C, Lc, nchunk;
   const float *k, *v, *u, *w;
   h1* r;
-  const float *aa, *bb, *pp;  // state before the sequence
+  const float *aa, *bb, *pp;  // state before the sequence (read by pass 1 only; may alias aa_out / bb_out / pp_out)
   float *la, *lb, *lp;        // [nchunk][C] local end states (pass 1)
-  float *sa, *sb, *sp;        // [nchunk][C] state at the start of each chunk (pass 2)
+  float *sa, *sb, *sp;        // [nchunk][C] state at the start of each chunk (row 0: pass 1; the rest: the serial pass)
   float *aa_out, *bb_out, *pp_out;
 };
 
@@ -248,6 +248,14 @@ __global__ __launch_bounds__(256) void wkv4_local_kernel(Wkv4Seq a) {
   a.la[o] = aa;
   a.lb[o] = bb;
   a.lp[o] = pp;
+  // The state before the sequence is copied into chunk 0's start-state slot.  The later passes read it
+  // from there, never from aa / bb / pp: the last chunk of the apply pass writes aa_out / bb_out / pp_out,
+  // which may be the same buffers, while chunks that were scheduled later have not started yet.
+  if (ch == 0) {
+    a.sa[c] = a.aa[c];
+    a.sb[c] = a.bb[c];
+    a.sp[c] = a.pp[c];
+  }
 }
 
 // The serial pass over the chunks.  A channel's step needs three values per chunk; they are read
@@ -258,7 +266,7 @@ __global__ __launch_bounds__(64) void wkv4_carry_kernel(Wkv4Seq a) {
   if (c >= a.C) return;
   constexpr int PF = 8;
   const float w = a.w[c];
-  float aa = a.aa[c], bb = a.bb[c], pp = a.pp[c];
+  float aa = a.sa[c], bb = a.sb[c], pp = a.sp[c];  // the incoming state, left there by wkv4_local_kernel
   for (int ch0 = 0; ch0 < a.nchunk; ch0 += PF) {
     float lp[PF], la[PF], lb[PF];
 #pragma unroll
@@ -305,7 +313,7 @@ __global__ __launch_bounds__(256) void wkv4_apply_kernel(Wkv4Seq a) {
   float aa, bb, pp;
   if constexpr (CARRY) {
     constexpr int PF = 8;
-    aa = a.aa[c], bb = a.bb[c], pp = a.pp[c];
+    aa = a.sa[c], bb = a.sb[c], pp = a.sp[c];  // the incoming state, left there by wkv4_local_kernel
     const float pdw = (float)a.Lc * w;  // every chunk before this one is a full chunk
     for (int j0 = 0; j0 < ch; j0 += PF) {
       float lp[PF], la[PF], lb[PF];
@@ -706,9 +714,14 @@ extern "C" int frhip_att_seq_v4(int T, int C, const void* x, const void* sx, con
   q.T = T; q.C = C;
   q.Lc = pick_chunk(T, (C + 255) / 256);
   // FRHIP_WKV4_SERIAL_CARRY=1: the chunk start states from a serial pass of their own (same bits)
-  static const bool serial_carry = getenv("FRHIP_WKV4_SERIAL_CARRY") != nullptr;
-  // a chunk composes the local states of all chunks before it: half as many, twice as long chunks
-  // (32 of 32 steps at T = 1024) cost the scans less than they save the composition
+  static const bool force_serial = getenv("FRHIP_WKV4_SERIAL_CARRY") != nullptr;
+  // Without the serial pass a chunk composes the local states of all chunks before it, nchunk / 2 compositions
+  // on average against Lc steps of its own: quadratic in T.  Beyond kComposeMaxChunks chunks of 32 steps
+  // (T > 4096) the serial pass takes over.
+  constexpr int kComposeMaxChunks = 128;
+  const bool serial_carry = force_serial || (T + 31) / 32 > kComposeMaxChunks;
+  // half as many, twice as long chunks (32 of 32 steps at T = 1024) cost the scans less than they save
+  // the composition
   if (!serial_carry && q.Lc < 32 && T >= 512) q.Lc = 32;
   q.nchunk = (T + q.Lc - 1) / q.Lc;
   q.k = w.f0; q.v = w.f1; q.u = t_first; q.w = t_decay; q.r = w.m3;

@@ -5,12 +5,18 @@
 //   small (<= 1 MiB): rounded to a power of two and served from per-class free lists;
 //     classes are refilled by carving 2 MiB slabs, so thousands of [C]-sized activation
 //     vectors cost a handful of hipMalloc calls;
-//   large: rounded to 2 MiB and served best-fit from a size-ordered pool of whole
-//     device allocations (weights, [T, F] prefill activations).
-// Memory is returned to the driver only by Trim().  All device work of the backend is
-// issued on one stream, so a block handed out again is ordered after its last use.
+//   large: rounded to 2 MiB and served best-fit from the free blocks of the driver
+//     allocations made so far ("segments": weights, [T, F] prefill activations).  A free
+//     block that is at least twice the request, or would leave 128 MiB or more unused, is
+//     split and its tail stays free (kernels/cuda/allocator.cpp:267-268); a released block
+//     merges with free neighbours of its segment (kernels/cuda/allocator.cpp:449-459), so
+//     prompts of changing length keep being served from the memory of the longest one.
+// Memory is returned to the driver only by Trim() (segments that are free as a whole).
+// All device work of the backend is issued on one stream, so a block handed out again is
+// ordered after its last use.
 #include <cstdio>
 #include <map>
+#include <set>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -29,6 +35,7 @@ public:
   static constexpr size_t kSmallMax = 1u << 20;
   static constexpr size_t kSlab = 2u << 20;
   static constexpr size_t kLargeRound = 2u << 20;
+  static constexpr size_t kSplitRemainder = 128u << 20;  // kernels/cuda/allocator.cpp:28 (kPieceSplitThreshold)
 
   void *DoAllocate(size_t size) override {
     stream();  // make sure the device is initialised
@@ -55,7 +62,7 @@ public:
     if (sz <= kSmallMax)
       _small[class_of(sz)].push_back(ptr);
     else
-      _large.emplace(sz, ptr);
+      free_large(static_cast<char *>(ptr));
   }
 
   // Give cached large blocks back to the driver; returns bytes released.
@@ -75,15 +82,54 @@ private:
     return c;
   }
 
-  size_t release_large_cache() {  // caller holds the mutex
+  // A block of a large segment.  Blocks of one segment tile it without gaps, in address order.
+  struct Block {
+    size_t size;
+    char *segment;  // start of the driver allocation this block is part of
+    bool free;
+  };
+  using BlockMap = std::map<char *, Block>;
+
+  // Release every segment that is one free block again; caller holds the mutex.
+  size_t release_large_cache() {
     size_t freed = 0;
-    for (auto &kv : _large) {
-      frhip_free(kv.second);
-      freed += kv.first;
+    for (auto it = _blocks.begin(); it != _blocks.end();) {
+      const auto seg = _segments.find(it->first);
+      if (it->second.free && seg != _segments.end() && seg->second == it->second.size) {
+        _free_by_size.erase({it->second.size, it->first});
+        frhip_free(it->first);
+        freed += it->second.size;
+        _segments.erase(seg);
+        it = _blocks.erase(it);
+      } else {
+        ++it;
+      }
     }
-    _large.clear();
     _reserved -= freed;
     return freed;
+  }
+
+  // Mark a large block free and merge it with free neighbours of the same segment.
+  void free_large(char *ptr) {
+    auto it = _blocks.find(ptr);
+    if (it == _blocks.end()) return;
+    it->second.free = true;
+    auto next = std::next(it);
+    if (next != _blocks.end() && next->second.free && next->second.segment == it->second.segment) {
+      _free_by_size.erase({next->second.size, next->first});
+      it->second.size += next->second.size;
+      _blocks.erase(next);
+    }
+    if (it != _blocks.begin()) {
+      auto prev = std::prev(it);
+      if (prev->second.free && prev->second.segment == it->second.segment) {
+        _free_by_size.erase({prev->second.size, prev->first});
+        prev->second.size += it->second.size;
+        _blocks.erase(it);
+        it = prev;
+      }
+    }
+    _free_by_size.insert({it->second.size, it->first});
   }
 
   void *raw(size_t bytes) {
@@ -113,27 +159,36 @@ private:
 
   void *alloc_large(size_t size) {
     const size_t rounded = (size + kLargeRound - 1) / kLargeRound * kLargeRound;
-    auto it = _large.lower_bound(rounded);
-    void *p = nullptr;
-    size_t got = rounded;
-    // reuse a cached block unless it would waste more than half of itself
-    if (it != _large.end() && it->first <= 2 * rounded) {
-      p = it->second;
-      got = it->first;
-      _large.erase(it);
+    BlockMap::iterator blk = _blocks.end();
+    auto fit = _free_by_size.lower_bound({rounded, nullptr});  // best fit: the smallest free block that is large enough
+    if (fit != _free_by_size.end()) {
+      blk = _blocks.find(fit->second);
+      _free_by_size.erase(fit);
     } else {
-      p = raw(rounded);
-      if (!p && release_large_cache() > 0) p = raw(rounded);  // last resort: release the cache and retry once
+      char *p = static_cast<char *>(raw(rounded));
+      if (!p && release_large_cache() > 0) p = static_cast<char *>(raw(rounded));  // last resort: release the cache and retry once
+      if (!p) return nullptr;
+      _segments[p] = rounded;
+      blk = _blocks.emplace(p, Block{rounded, p, true}).first;
     }
-    if (!p) return nullptr;
-    _live[p] = got;
-    _in_use += got;
-    return p;
+    Block &b = blk->second;
+    if (b.size >= 2 * rounded || b.size - rounded >= kSplitRemainder) {  // the tail stays in the pool
+      char *tail = blk->first + rounded;
+      _blocks.emplace(tail, Block{b.size - rounded, b.segment, true});
+      _free_by_size.insert({b.size - rounded, tail});
+      b.size = rounded;
+    }
+    b.free = false;
+    _live[blk->first] = b.size;
+    _in_use += b.size;
+    return blk->first;
   }
 
   std::mutex _mu;
   std::unordered_map<int, std::vector<void *>> _small;
-  std::multimap<size_t, void *> _large;
+  BlockMap _blocks;                                  // every block of every large segment, by address
+  std::set<std::pair<size_t, char *>> _free_by_size;  // the free ones, by size then address
+  std::map<char *, size_t> _segments;                // driver allocations of the large regime: start -> bytes
   std::unordered_map<void *, size_t> _live;
   size_t _reserved = 0, _in_use = 0, _driver_calls = 0;
 };

@@ -234,6 +234,54 @@ def test_allocator_reuses_memory_and_decoding_makes_no_driver_calls():
     assert u4 < u3 and r4 == r3         # the model's memory went back to the pool, not to the driver
 
 
+def test_allocator_prompts_of_changing_length_are_served_from_the_first_ones_memory():
+    """Large blocks are split for smaller requests and merge again when released
+    (kernels/cuda/allocator.cpp:267-268, 449-459): after the longest prompt no later, shorter one
+    makes the pool grow."""
+    m = fr.Model("synthetic:v=4,L=4,C=1024,F=4096,V=4096,seed=5", "hip fp16")
+    g = np.random.default_rng(2)
+    m.run([int(t) for t in g.integers(0, 4096, 1024)])
+    r0, u0, c0 = fr.allocator_stats()
+    for T in (700, 333, 1000, 1024, 64, 1001):
+        m.reset()
+        m.run([int(t) for t in g.integers(0, 4096, T)])
+        r, u, c = fr.allocator_stats()
+        assert (r, c) == (r0, c0), "a prompt of %d tokens after one of 1024 grew the pool by %d bytes" % (T, r - r0)
+    m.close()
+
+
+def test_allocator_splits_large_blocks_and_merges_them_again():
+    h = fr.host()
+    fr.init()
+    h.fr_allocator_trim()
+    MB = 1 << 20
+    big = h.fr_hip_alloc(64 * MB)
+    assert big
+    calls = fr.allocator_stats()[2]
+    h.fr_hip_free(big)
+    a = h.fr_hip_alloc(16 * MB)          # at least twice the request: the block is split, the front handed out
+    b = h.fr_hip_alloc(16 * MB)          # from the tail
+    c = h.fr_hip_alloc(30 * MB)          # the remaining 32 MiB are less than twice 30: handed out whole
+    assert (a, b, c) == (big, big + 16 * MB, big + 32 * MB) and fr.allocator_stats()[2] == calls
+    used = fr.allocator_stats()[1]
+    h.fr_hip_free(b)                     # a hole between two live blocks
+    assert fr.allocator_stats()[1] == used - 16 * MB
+    d = h.fr_hip_alloc(10 * MB)          # best fit: the 16 MiB hole, not split (10 < 16 < 20)
+    assert d == b and fr.allocator_stats()[1] == used
+    for p in (a, c, d):
+        h.fr_hip_free(p)
+    again = h.fr_hip_alloc(64 * MB)      # the three blocks merged back into the segment
+    assert again == big and fr.allocator_stats()[2] == calls
+    h.fr_hip_free(again)
+    # a segment with a live block is not released; once it is free as a whole, it is
+    a = h.fr_hip_alloc(8 * MB)
+    assert a == big
+    reserved = fr.allocator_stats()[0]
+    assert h.fr_allocator_trim() == 0 and fr.allocator_stats()[0] == reserved
+    h.fr_hip_free(a)
+    assert h.fr_allocator_trim() >= 64 * MB
+
+
 def test_allocator_alignment_reuse_trim_and_out_of_memory():
     h = fr.host()
     fr.init()

@@ -201,6 +201,38 @@ def test_att_seq_v4(T, C_, quant, fresh):
     assert np.abs(po_.numpy() - ref[4]).max() < 30  # offsets stay in a sane range
 
 
+@pytest.mark.parametrize("T,C_", [(1024, 2048), (700, 512), (5000, 256)])  # 5000: beyond 128 chunks of 32 steps, the scan's serial pass
+def test_att_seq_v4_state_updated_in_place_equals_separate_outputs(T, C_):
+    """The header allows aa_out / bb_out / pp_out to be the buffers of aa / bb / pp (as frhip_att_one_v4 does).
+    The scan's last chunk writes them while other chunks may not have started: every pass must take the
+    incoming state from the copy the first pass makes.  Bit for bit the same as with separate outputs."""
+    x, sx = h(rng.standard_normal((T, C_)) * 2), h(rng.standard_normal(C_))
+    aa, bb, pp = _state_v4(C_, False)
+    ln_w, ln_b = _common(C_)
+    mixes = [h(rng.uniform(0, 1, C_)) for _ in range(3)]
+    td = (-np.exp(rng.uniform(-5, 1, C_))).astype(np.float32)
+    tf = rng.uniform(-1, 1, C_).astype(np.float32)
+    pairs = [make_weight(h(rng.standard_normal((C_, C_)) * 0.02), False) for _ in range(4)]
+    ws_, refs = [p[0] for p in pairs], [p[1] for p in pairs]
+    ws = DevBuf(L().frhip_seq_workspace_bytes(T, C_, 4 * C_))
+    dx, dsx = keep(x), keep(sx)
+    consts = [keep(a).ptr for a in (ln_w, ln_b, *mixes, td, tf)]
+    results = []
+    for in_place in (False, True):
+        st = [dev(aa), dev(bb), dev(pp)]
+        outs = st if in_place else [DevBuf.empty(C_, np.float32) for _ in range(3)]
+        x_out, xx_out = DevBuf.empty((T, C_), np.float16), DevBuf.empty(C_, np.float16)
+        fr.check(L().frhip_att_seq_v4(T, C_, dx.ptr, dsx.ptr, st[0].ptr, st[1].ptr, st[2].ptr, *consts,
+                                      *[w.ref for w in ws_], x_out.ptr, xx_out.ptr, outs[0].ptr, outs[1].ptr, outs[2].ptr,
+                                      ws.ptr, None))
+        results.append([x_out.numpy(), xx_out.numpy()] + [o.numpy() for o in outs])
+    for sep, inp in zip(*results):
+        assert np.array_equal(sep, inp)
+    if T == 5000:  # the long prompt against the oracle as well (the serial pass is otherwise only reached by a switch)
+        ref = po.att_seq_v4_f16(x, sx, aa, bb, pp, ln_w, ln_b, *mixes, td, tf, *refs)
+        assert_close_f16(results[0][0], ref[0], max_ulp=3, max_frac=0.1, what="x_out, T = 5000")
+
+
 @pytest.mark.parametrize("T,C_,H_", [(48, 512, 8), (512, 2560, 40), (1, 512, 8), (77, 512, 8), (3000, 512, 8), (40, 2560, 40)])  # (40, 2560, 40): k,v,r,g of a short prompt in one split launch
 @pytest.mark.parametrize("quant", [False, True])
 def test_att_seq_v5_2(T, C_, H_, quant):
