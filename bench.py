@@ -3,9 +3,11 @@
 
     python bench.py [--gpus 1] [--steps 512] [--warmup 16] [--dtype fp16|int8]
 
-A "step" is one decoded token: rwkv::Model::Run(id) through the `hip` device (fused kernels
-replayed as a HIP graph), the fp32 logits copied to the host, and the host-side argmax that
-picks the next token -- the loop chat.cpp runs with top_k = 1.  Weights are random-init of
+A "step" is one decoded token of the loop the reference's chat.cpp:56-92 / bench_model.cpp:7-8 run: one
+rwkv::Model::Run(id) through the `hip` device (fused kernels replayed as a HIP graph) that returns the fp32
+logits on the host, the greedy choice of the next token, the next Run -- one host wait per token
+(FR_HIP_GREEDY_ON_HOST=1).  The same loop kept on the device (fr_greedy_decode's default, which the reference's
+API does not have) is reported beside it in `extra`.  Weights are random-init of
 the named architecture (there are no checkpoints here) and are resident in HBM before the
 timed region starts.
 
@@ -226,8 +228,12 @@ def rwkv5_extra(fr):
             best = min(best, time.perf_counter() - t0)
     finally:
         del os.environ["FR_HIP_SEQ_IMAGE"]
-    m.greedy(int(np.argmax(lg)), 16)
-    _, secs = m.greedy(17, 256)
+    os.environ["FR_HIP_GREEDY_ON_HOST"] = "1"  # Model::Run per token, as the headline
+    try:
+        m.greedy(int(np.argmax(lg)), 16)
+        _, secs = m.greedy(17, 256)
+    finally:
+        del os.environ["FR_HIP_GREEDY_ON_HOST"]
     # the same prompt with the binary16 image of the uint8 weights kept on the device (FR_HIP_SEQ_IMAGE=1, the default
     # on a device of this size: 2 more bytes per weight, no expansion per call); the first pass makes the images and is not timed
     os.environ["FR_HIP_SEQ_IMAGE"] = "1"
@@ -243,20 +249,27 @@ def rwkv5_extra(fr):
         del os.environ["FR_HIP_SEQ_IMAGE"]
     assert np.array_equal(lg, lg2), "kept binary16 image changed the logits"
     m.close()
-    wbytes = 32 * 85196800 + 167772160  # uint8 codes of every matrix, once per token
-    return {"rwkv5_3b_int8_prefill_T512_ms": round(kept * 1e3, 2), "rwkv5_3b_int8_prefill_tok_s": round(512 / kept, 1),
-            "rwkv5_3b_int8_prefill_T512_expanded_per_call_ms": round(best * 1e3, 2),
+    # Algorithmic bytes per token: the uint8 codes of every matrix once, their offsets / ranges, the [H, 64, 64] fp32
+    # state of every layer read and written, activation vectors in and out.
+    C5, F5, Lr = 2560, 8960, 32
+    mats = [(C5, C5)] * 5 + [(C5, F5), (F5, C5), (C5, C5)]
+    per_layer = sum(k * n + 4 * (k + n) + 2 * k + 2 * n for k, n in mats) + 2 * 4 * C5 * 64
+    abytes = Lr * per_layer + C5 * V_ + 4 * (C5 + V_) + 2 * C5 + 4 * V_
+    return {"rwkv5_3b_int8_prefill_T512_ms": round(best * 1e3, 2), "rwkv5_3b_int8_prefill_tok_s": round(512 / best, 1),
+            "rwkv5_3b_int8_prefill_T512_kept_fp16_image_ms": round(kept * 1e3, 2),
             "rwkv5_3b_int8_decode_tok_s": round(256 / secs, 1),
-            "rwkv5_3b_int8_decode_weight_GBs": round(wbytes * 256 / secs / 1e9, 1)}
+            "rwkv5_3b_int8_decode_bytes_per_token": abytes,
+            "rwkv5_3b_int8_decode_GBs": round(abytes * 256 / secs / 1e9, 1),
+            "rwkv5_3b_int8_decode_frac_of_hbm_peak": round(abytes * 256 / secs / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 def cpu_baseline(seconds_budget=20.0):
-    """The oracle's fp32 one-token forward on the host cores (OpenMP over output columns), on
-    the same architecture with the depth cut to 2 layers + head to bound the run; the
-    per-token time is scaled to 24 layers by the measured per-layer time."""
+    """The oracle's fp32 one-token forward on the host cores (OpenMP over output columns): the whole
+    24-layer 1.5B shape (6 GB of fp32 weights; every layer has weight arrays of its own, filled from one
+    random block, so that no layer finds its weights in a cache), greedy tokens, for a bounded number of
+    tokens -- on all threads the runtime gives, and on one."""
     import pyoracle as po
     rng = np.random.default_rng(1)
-    Ls = 2
 
     def mat(k, n):
         return (rng.standard_normal((k, n), dtype=np.float32) * 0.02)
@@ -264,36 +277,40 @@ def cpu_baseline(seconds_budget=20.0):
     def vec(lo, hi):
         return rng.uniform(lo, hi, C_).astype(np.float32)
 
+    block = [np.ones(C_, np.float32), np.zeros(C_, np.float32), vec(0, 1), vec(0, 1), vec(0, 1),
+             -np.exp(vec(-5, 1)), vec(-1, 1), mat(C_, C_), mat(C_, C_), mat(C_, C_), mat(C_, C_),
+             np.ones(C_, np.float32), np.zeros(C_, np.float32), vec(0, 1), vec(0, 1), mat(C_, F_), mat(F_, C_),
+             mat(C_, C_)]
     params = []
-    for _ in range(Ls):
-        params += [np.ones(C_, np.float32), np.zeros(C_, np.float32), vec(0, 1), vec(0, 1), vec(0, 1),
-                   -np.exp(vec(-5, 1)), vec(-1, 1), mat(C_, C_), mat(C_, C_), mat(C_, C_), mat(C_, C_),
-                   np.ones(C_, np.float32), np.zeros(C_, np.float32), vec(0, 1), vec(0, 1), mat(C_, F_), mat(F_, C_),
-                   mat(C_, C_)]
+    for _ in range(L_):
+        params += [a.copy() for a in block]
     params += [np.ones(C_, np.float32), np.zeros(C_, np.float32), mat(C_, V_)]
     emb = rng.standard_normal((1024, C_), dtype=np.float32)
-    full = po.Model(4, po.F32, Ls, C_, F_, 0, V_, params, emb)
-    shallow = po.Model(4, po.F32, 1, C_, F_, 0, V_, params[:18] + params[-3:], emb)
+    model = po.Model(4, po.F32, L_, C_, F_, 0, V_, params, emb)
 
-    def per_token(m, budget):
-        m.run(1)
+    def per_token(budget, most):
+        tok = int(np.argmax(model.run(1))) % 1024
         n, t0 = 0, time.perf_counter()
         while True:
-            m.run(n % 1024)
+            tok = int(np.argmax(model.run(tok))) % 1024
             n += 1
             dt = time.perf_counter() - t0
-            if dt > budget or n >= 64:
+            if dt > budget or n >= most:
                 return dt / n, n
 
-    t2, n2 = per_token(full, seconds_budget * 0.6)
-    t1, n1 = per_token(shallow, seconds_budget * 0.4)
-    per_layer = max(t2 - t1, 1e-9)
-    head_t = max(t1 - per_layer, 0.0)
-    t24 = L_ * per_layer + head_t
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": round(1.0 / t24, 3), "unit": "tok/s", "cores": cores, "kind": "port",
-            "sample": "oracle fp32 one-token forward, 2-layer and 1-layer slices of the 1.5B shape + 65536 head, "
-                      "%d+%d tokens timed; per-layer time x24 + head" % (n2, n1)}
+    t_all, n_all = per_token(seconds_budget * 0.5, 128)
+    # the same on one thread (the oracle's loops are OpenMP-parallel: the thread count is the runtime's to set)
+    gomp = C.CDLL("libgomp.so.1")
+    gomp.omp_set_num_threads(1)
+    try:
+        t_one, n_one = per_token(seconds_budget * 0.5, 8)
+    finally:
+        gomp.omp_set_num_threads(cores)
+    return {"value": round(1.0 / t_all, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "single_thread_value": round(1.0 / t_one, 3), "nproc": os.cpu_count(),
+            "sample": "oracle fp32 one-token forward of the whole 24-layer 1.5B shape (vocab 65536), greedy: "
+                      "%d tokens timed on %d threads, %d tokens on one thread" % (n_all, cores, n_one)}
 
 
 def probe_mfma(fr, iters=20000, reps=3):
@@ -463,12 +480,24 @@ def main():
     build_s = time.perf_counter() - t0
     print("[bench] model built in %.1f s: %s" % (build_s, cfg["workload"]), file=sys.stderr, flush=True)
 
-    model.greedy(0, 2)  # set-up, like the build: the first greedy call captures the plan's graphs
+    # the timed loop: Model::Run per token with the host between the tokens
+    os.environ["FR_HIP_GREEDY_ON_HOST"] = "1"
+    try:
+        model.greedy(0, 2)  # set-up, like the build: the first call captures the plan's graphs
+        model.greedy(0, args.warmup)
+        fr.check(fr.lib().frhip_device_sync())
+        toks, secs = model.greedy(17, args.steps)
+        fr.check(fr.lib().frhip_device_sync())
+    finally:
+        del os.environ["FR_HIP_GREEDY_ON_HOST"]
+    # the same tokens with the greedy choice kept on the device (no host between the tokens)
+    model.reset()
+    model.greedy(0, 2)
     model.greedy(0, args.warmup)
-    fr.check(fr.lib().frhip_device_sync())
-    toks, secs = model.greedy(17, args.steps)
+    toks_dev, secs_dev = model.greedy(17, args.steps)
     fr.check(fr.lib().frhip_device_sync())
     model.close()
+    assert np.array_equal(toks, toks_dev), "the device-side greedy chain chose other tokens than the loop of Run calls"
     ms_per_step = 1e3 * secs / args.steps
     tok_s = args.steps / secs
 
@@ -488,10 +517,10 @@ def main():
         "dtype": "f16" if args.dtype == "fp16" else "u8 weights, f16 activations, f32 accumulate",
         "data": "synthetic (random-init weights, greedy token ids)",
         "config": {"workload": cfg["workload"], "strategy": cfg["strategy"], "steps": args.steps,
-                   "host_loop": "fr_greedy_decode: one graph per token (two tokens per graph where the parity allows), queued back to back; "
-                                "each token's first kernel takes its token from the 64 per-slice arg-max pairs of the token before; every token's "
-                                "logits still go to pinned host memory; the host waits once per batch of at most 1023 tokens "
-                                "(extra.*_host_in_loop: Model::Run + host reduction of the pairs, one wait per token)"},
+                   "host_loop": "Model::Run per token (chat.cpp:56-92, bench_model.cpp:7-8): one graph launch and one stream wait per "
+                                "token, the logits in host memory after every token, the greedy token from the 64 per-slice arg-max "
+                                "pairs the graph leaves beside them (extra.*_device_side_greedy_chain: the same tokens with the choice "
+                                "kept on the device, the host waiting once per batch of tokens)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "row-streaming matrix-vector kernels (att_front/att_out/ffn_front/ffn_out/head), "
@@ -500,36 +529,41 @@ def main():
                      "avg_launch_us": round(1e3 * kernel_ms / n_launch, 3)},
         "roofline_tok_s": round(1.0 / (abytes / (HBM_PEAK_GBS * 1e9)), 1),
     }
+    dev_chain = {args.dtype + "_decode_tok_s_device_side_greedy_chain": round(args.steps / secs_dev, 2)}
+    if args.no_extras:
+        out["extra"] = dev_chain
     if not args.no_extras:
-        extra = {}
+        extra = dict(dev_chain)
         other = "int8" if args.dtype == "fp16" else "fp16"
         ocfg = CONFIGS[other]
         om = fr.Model(ocfg["spec"], ocfg["strategy"])
+        os.environ["FR_HIP_GREEDY_ON_HOST"] = "1"
+        try:
+            om.greedy(0, args.warmup)
+            _, osecs = om.greedy(17, args.steps)
+        finally:
+            del os.environ["FR_HIP_GREEDY_ON_HOST"]
+        om.reset()
         om.greedy(0, args.warmup)
-        _, osecs = om.greedy(17, args.steps)
+        _, osecs_dev = om.greedy(17, args.steps)
         om.close()
         okms, _ = measure_kernels(fr, ocfg)
         ob = algorithmic_bytes_per_token(ocfg["wbytes"])
         extra[other + "_decode_tok_s"] = round(args.steps / osecs, 2)
+        extra[other + "_decode_tok_s_device_side_greedy_chain"] = round(args.steps / osecs_dev, 2)
         extra[other + "_gemv_GBs"] = round(ob / (okms * 1e-3) / 1e9, 1)
         extra[other + "_gemv_frac_of_hbm_peak"] = round(ob / (okms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         # companions of the headline: the same loop over 512 steps when the run was shorter, and with
         # Model::Run returning a tensor of its own (FR_HIP_OWNED_LOGITS=1) instead of a view of pinned memory
         if args.dtype == "fp16":
-            if args.steps < 512:
-                lm = fr.Model(cfg["spec"], cfg["strategy"])
-                lm.greedy(0, 16)
-                _, lsecs = lm.greedy(17, 512)
-                lm.close()
-                extra["fp16_decode_tok_s_512_steps"] = round(512 / lsecs, 2)
-            # the loop the reference's chat.cpp:56-92 runs: Model::Run, arg-max on the host, Model::Run
             os.environ["FR_HIP_GREEDY_ON_HOST"] = "1"
             try:
-                hm = fr.Model(cfg["spec"], cfg["strategy"])
-                hm.greedy(0, 16)
-                _, hsecs = hm.greedy(17, 512)
-                hm.close()
-                extra["fp16_decode_tok_s_host_in_loop"] = round(512 / hsecs, 2)
+                if args.steps < 512:
+                    lm = fr.Model(cfg["spec"], cfg["strategy"])
+                    lm.greedy(0, 16)
+                    _, lsecs = lm.greedy(17, 512)
+                    lm.close()
+                    extra["fp16_decode_tok_s_512_steps"] = round(512 / lsecs, 2)
                 os.environ["FR_HIP_OWNED_LOGITS"] = "1"
                 wm = fr.Model(cfg["spec"], cfg["strategy"])
                 wm.greedy(0, 16)
@@ -538,7 +572,7 @@ def main():
             finally:
                 os.environ.pop("FR_HIP_OWNED_LOGITS", None)
                 del os.environ["FR_HIP_GREEDY_ON_HOST"]
-            extra["fp16_decode_tok_s_host_in_loop_owned_logits"] = round(512 / wsecs, 2)
+            extra["fp16_decode_tok_s_owned_logits"] = round(512 / wsecs, 2)
         extra.update(prefill_extra(fr))
         extra.update(rwkv5_extra(fr))
         extra.update(probe_bandwidth(fr))

@@ -259,10 +259,13 @@ def host():
         h.fr_sampler_sample.argtypes = [_vp, _vp, _i, C.c_float, _i, C.c_float]
         h.fr_sample_decode.restype = C.c_longlong
         h.fr_sample_decode.argtypes = [_vp, _vp, _i, _i, C.c_float, _i, C.c_float, _vp]
+        h.fr_chat_decode.restype = C.c_longlong
+        h.fr_chat_decode.argtypes = [_vp, _vp, _i, _i, C.c_float, _i, C.c_float, C.c_float, C.c_float, C.c_float, _vp]
         h.fr_model_reset.argtypes = [_vp]
         h.fr_model_save_state.argtypes = [_vp, C.c_char_p]
         h.fr_model_load_state.argtypes = [_vp, C.c_char_p]
         h.fr_model_get_state.argtypes = [_vp, _i, _i, _vp, _i]
+        h.fr_model_set_state.argtypes = [_vp, _i, _i, _vp, _i]
         h.fr_model_snapshot.restype = _vp
         h.fr_model_snapshot.argtypes = [_vp]
         h.fr_model_restore.argtypes = [_vp, _vp]
@@ -375,6 +378,11 @@ class Model:
         n = self._chk(self._h.fr_model_get_state(self._m, layer, index, buf.ctypes.data, buf.size))
         return buf[:n].view(dtype).copy()
 
+    def set_state(self, layer, index, a):
+        """Replace one state tensor by a numpy array of the same size and dtype (what LoadStateFile does per tensor)."""
+        a = np.ascontiguousarray(a)
+        self._chk(self._h.fr_model_set_state(self._m, layer, index, a.ctypes.data, a.nbytes))
+
     def snapshot(self):
         """A copy of Model::states() (shares storage, as `auto s = model.states();` does); give it to restore()."""
         s = self._h.fr_model_snapshot(self._m)
@@ -389,11 +397,17 @@ class Model:
     def free_snapshot(self, snap):
         self._h.fr_snapshot_free(snap)
 
-    def generate(self, sampler, first_id, steps, temperature=1.0, top_k=0, top_p=1.0):
-        """chat.cpp:56-92 without its penalties, in C++; returns (token ids, seconds)."""
+    def generate(self, sampler, first_id, steps, temperature=1.0, top_k=0, top_p=1.0, presence_penalty=0.0,
+                 frequency_penalty=0.0, penalty_decay=1.0):
+        """The generation loop of chat.cpp:56-92 in C++ (its penalties are 0.8, 0.8 and 0.996, chat.cpp:22-24);
+        returns (token ids, seconds)."""
         out = np.empty(steps, np.int32)
-        us = self._h.fr_sample_decode(self._m, sampler._s, int(first_id), int(steps), temperature, top_k, top_p,
-                                      out.ctypes.data)
+        if presence_penalty or frequency_penalty:
+            us = self._h.fr_chat_decode(self._m, sampler._s, int(first_id), int(steps), temperature, top_k, top_p,
+                                        presence_penalty, frequency_penalty, penalty_decay, out.ctypes.data)
+        else:
+            us = self._h.fr_sample_decode(self._m, sampler._s, int(first_id), int(steps), temperature, top_k, top_p,
+                                          out.ctypes.data)
         if us < 0:
             raise FrhipError(self._h.fr_last_error().decode())
         return out, us * 1e-6

@@ -4,6 +4,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <map>
 #include <string>
 
 #include "kernels/hip/context.h"
@@ -125,8 +126,38 @@ int fr_sampler_sample(void *s, const float *logits, int n, float temperature, in
   return guarded([&]() { return static_cast<rwkv::Sampler *>(s)->Sample(logits, n, temperature, top_k, top_p); });
 }
 
-// The generation loop of chat.cpp:56-92 without its penalties: feed first_id, sample, feed
-// the sample, `steps` times.  Returns the elapsed microseconds, or -1.
+// The generation loop of chat.cpp:56-92: feed first_id, adjust the host logits by the repetition
+// penalties, sample, feed the sample, `steps` times.  As there, every token drawn so far has
+// `frequency_penalty * count + presence_penalty` subtracted from its logit before the draw, in the order of the
+// occurrence map, and its count is then multiplied by `penalty_decay` (chat.cpp:57-62); the drawn token's
+// count goes up by one (chat.cpp:77).  The reference's values are 0.8, 0.8 and 0.996 (chat.cpp:22-24).  The
+// adjustments its question-and-answer mode makes to two token ids of its own vocabulary (chat.cpp:63-74) belong
+// to that front end and are not made here.  Returns the elapsed microseconds, or -1.
+long long fr_chat_decode(void *m, void *sampler, int first_id, int steps, float temperature, int top_k, float top_p,
+                         float presence_penalty, float frequency_penalty, float penalty_decay, int *out_ids) {
+  return guarded([&]() -> long long {
+    auto *model = static_cast<rwkv::Model *>(m);
+    auto *smp = static_cast<rwkv::Sampler *>(sampler);
+    std::map<int, float> occurrences;
+    int id = first_id;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; i++) {
+      // the logits are adjusted in place: Run's result is the caller's to change until the next-but-one call
+      rwkv::Tensor out = rwkv::Copy(model->Run(id), rwkv::Device::kCPU);
+      float *logits = out.data_ptr<float>();
+      for (auto &[tok, count] : occurrences) {
+        logits[tok] -= frequency_penalty * count + presence_penalty;
+        count *= penalty_decay;
+      }
+      id = smp->Sample(out, temperature, top_k, top_p);
+      occurrences[id]++;
+      out_ids[i] = id;
+    }
+    return std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count();
+  });
+}
+
+// The same loop without penalties.
 long long fr_sample_decode(void *m, void *sampler, int first_id, int steps, float temperature, int top_k,
                            float top_p, int *out_ids) {
   return guarded([&]() -> long long {
@@ -193,6 +224,20 @@ int fr_model_get_state(void *m, int layer, int index, void *out, int capacity) {
     if (n > capacity) throw FRException("state buffer too small");
     std::memcpy(out, c.data_ptr(), static_cast<size_t>(n));
     return n;
+  });
+}
+
+// Replace state tensor (layer, index) by `nbytes` raw bytes from the host (same shape and dtype), as
+// LoadStateFile does for every tensor of a file (model.cpp:117-143).
+int fr_model_set_state(void *m, int layer, int index, const void *data, int nbytes) {
+  return guarded([&]() {
+    auto *model = static_cast<rwkv::Model *>(m);
+    rwkv::Tensor &dst = model->states().at(layer).at(index);
+    if (static_cast<size_t>(nbytes) != dst.nbytes()) throw FRException("state tensor size mismatch");
+    rwkv::Tensor t = rwkv::Tensor::Empty(dst.shape(), dst.dtype(), rwkv::Device::kCPU);
+    std::memcpy(t.data_ptr(), data, static_cast<size_t>(nbytes));
+    dst = rwkv::Copy(t, dst.device());
+    return 0;
   });
 }
 

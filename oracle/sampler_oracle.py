@@ -70,3 +70,26 @@ def sample(logits, temperature, top_k, top_p, gen):
         if cumsum >= r:
             return order[i]
     raise RuntimeError("cumulative scan ended below the draw")
+
+
+class Penalties:
+    """The repetition penalties of the reference's generation loop (chat.cpp:22-24, 40, 57-62, 77), in the
+    loop's own arithmetic: before every draw, each token drawn so far (in ascending id order, the order of
+    the std::map) has `frequency * count + presence` subtracted from its fp32 logit, the product and the sum
+    evaluated in fp32, and its count is then multiplied by `decay`; the drawn token's count goes up by one."""
+
+    def __init__(self, presence=0.8, frequency=0.8, decay=0.996):
+        self.presence, self.frequency, self.decay = F(presence), F(frequency), F(decay)
+        self.count = {}
+
+    def apply(self, logits):
+        """Adjusts `logits` (fp32 array) in place and decays the counts (chat.cpp:57-62)."""
+        for tok in sorted(self.count):
+            c = self.count[tok]
+            logits[tok] = F(logits[tok] - F(F(self.frequency * c) + self.presence))
+            self.count[tok] = F(c * self.decay)
+        return logits
+
+    def drawn(self, tok):
+        """chat.cpp:77: `occurences[output_id]++`."""
+        self.count[tok] = F(self.count.get(tok, F(0)) + F(1))

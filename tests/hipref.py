@@ -53,30 +53,83 @@ def same_token_or_near_tie(lh, lo):
     return th == to or float(lo[to] - lo[th]) <= 2 * float(np.abs(lh - lo).max())
 
 
-def greedy_against_oracle(run_hip, run_oracle, prompt, steps, tol=2e-2, report=None, tag=""):
-    """The parity criterion: feed `prompt` token by token, then `steps` greedy steps; at every step the
-    logits agree within `tol` (max-abs) and the greedy tokens agree (or differ at a near-tie, see
-    same_token_or_near_tie; both sides then continue with the oracle's token).
-    Returns (worst max-abs logit difference, number of near-tie steps)."""
+def binary16_spacing(v):
+    """Distance between neighbouring binary16 values at magnitude |v| (normal range)."""
+    return float(np.exp2(np.floor(np.log2(max(abs(float(v)), 2.0 ** -14))) - 10))
+
+
+class StateSynchronised:
+    """A second `hip` model that is handed the oracle's recurrent state before every token, so that a step's
+    comparison measures what ONE step of the implementation adds: two binary16 pipelines that are not
+    bit-identical drift apart over many steps whatever the size of their first difference, and a free-running
+    comparison cannot tell that drift from an implementation error.  `per_layer` = state tensors per layer
+    (model.cpp:152-175: five for RWKV-4, three for RWKV-5)."""
+
+    def __init__(self, model, oracle_model, per_layer):
+        self.m, self.om, self.per = model, oracle_model, per_layer
+
+    def run(self, tok):
+        """Load the oracle's current state, then one token.  Call BEFORE the oracle runs the same token."""
+        for i, a in enumerate(self.om.state):
+            self.m.set_state(i // self.per, i % self.per, a)
+        return self.m.run(int(tok))
+
+
+def greedy_against_oracle(run_hip, run_oracle, prompt, steps, tol=2e-2, report=None, tag="", synced=None,
+                          max_swaps=None, stats=None):
+    """The parity criterion: feed `prompt` token by token, then `steps` greedy steps.
+
+    Free-running (`run_hip`): at every step the logits agree within `tol` (max-abs; None = not asserted here) and
+    the greedy tokens agree or differ at a near-tie (same_token_or_near_tie; both sides then continue with the
+    oracle's token); at most `max_swaps` such steps.
+
+    State-synchronised (`synced`, a StateSynchronised): the criterion as written, strictly -- at every step
+    max-abs <= 2e-2 and the same greedy token whenever the oracle's margin between its two largest logits
+    exceeds one binary16 spacing of the largest (logits are binary16 values: closer than that is a tie).
+
+    Returns (worst free-running max-abs difference, free-running steps with unequal tokens); `stats`, if given,
+    receives the state-synchronised figures as well."""
     import time
+    st = stats if stats is not None else {}
+    st.update(worst=0.0, swaps=0, sync_worst=0.0, sync_unequal=0, sync_steps=0)
+
+    def one(tok):
+        ls = synced.run(tok) if synced is not None else None  # before the oracle moves its state
+        return run_hip(int(tok)), run_oracle(int(tok)), ls
+
     for t in prompt:
-        lh, lo = run_hip(int(t)), run_oracle(int(t))
-    worst, swaps, t0 = 0.0, 0, time.time()
+        lh, lo, ls = one(t)
+    t0 = time.time()
     for step in range(steps):
         d = float(np.abs(lh - lo).max())
-        worst = max(worst, d)
+        st["worst"] = max(st["worst"], d)
         th, to = int(np.argmax(lh)), int(np.argmax(lo))
         if th != to:
             assert same_token_or_near_tie(lh, lo), "%s: greedy token differs at step %d (hip %d, oracle %d, oracle margin %g, |dlogit| %g)" % (
                 tag, step, th, to, float(lo[to] - lo[th]), d)
-            swaps += 1
-        lh, lo = run_hip(to), run_oracle(to)
+            st["swaps"] += 1
+        if ls is not None:
+            ds = float(np.abs(ls - lo).max())
+            st["sync_worst"] = max(st["sync_worst"], ds)
+            st["sync_steps"] += 1
+            assert ds <= 2e-2, "%s: state-synchronised step %d: |dlogit| %g" % (tag, step, ds)
+            ts = int(np.argmax(ls))
+            if ts != to:
+                margin = float(lo[to] - np.partition(lo, -2)[-2])
+                assert margin <= binary16_spacing(lo[to]), "%s: state-synchronised step %d: token %d, oracle %d, oracle margin %g" % (
+                    tag, step, ts, to, margin)
+                st["sync_unequal"] += 1
+        lh, lo, ls = one(to)
         if report and step % 32 == 31:
-            report("%s: %d steps, worst |dlogit| %.2e, %d near-tie swaps, %.0f s" % (tag, step + 1, worst, swaps, time.time() - t0))
+            report("%s: %d steps, worst |dlogit| %.2e, %d near-tie swaps%s, %.0f s" % (
+                tag, step + 1, st["worst"], st["swaps"],
+                "; state-synchronised: worst %.2e, %d ties" % (st["sync_worst"], st["sync_unequal"]) if synced is not None else "",
+                time.time() - t0))
     if tol is not None:
-        assert worst <= tol, "%s: worst |dlogit| %g" % (tag, worst)
-    assert swaps <= max(1, steps // 16), "%s: tokens differed at %d of %d steps" % (tag, swaps, steps)
-    return worst, swaps
+        assert st["worst"] <= tol, "%s: worst |dlogit| %g" % (tag, st["worst"])
+    limit = max(1, steps // 16) if max_swaps is None else max_swaps
+    assert st["swaps"] <= limit, "%s: tokens differed at %d of %d steps (limit %d)" % (tag, st["swaps"], steps, limit)
+    return st["worst"], st["swaps"]
 
 
 def make_weight(w_kn, quant=False):

@@ -341,6 +341,35 @@ def test_sampled_generation_follows_the_oracle_sampler(model_files):
     m.close()
 
 
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 1, 0.0), (1.2, 50, 0.9)])  # chat.cpp:76-77's own settings; a sampled run
+def test_generation_with_the_repetition_penalties_of_the_chat_loop(model_files, temperature, top_k, top_p):
+    """chat.cpp:56-92 with its presence / frequency penalties and their decay (0.8, 0.8, 0.996: chat.cpp:22-24):
+    the C++ loop on the hip model draws the tokens that the oracle's sampler draws from the same logits adjusted
+    by the oracle's statement of the penalties, and the penalties change what is drawn."""
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
+    import sampler_oracle as so
+    path, params, emb = model_files
+    m = fr.Model(path, "hip fp16")
+    steps = 48
+    toks, _ = m.generate(fr.Sampler(77), 5, steps, temperature=temperature, top_k=top_k, top_p=top_p,
+                         presence_penalty=0.8, frequency_penalty=0.8, penalty_decay=0.996)
+    m.reset()
+    plain, _ = m.generate(fr.Sampler(77), 5, steps, temperature=temperature, top_k=top_k, top_p=top_p)
+    assert not np.array_equal(toks, plain)
+    if top_k == 1:  # greedy: without penalties the device-side loop gives the same tokens, with them it is not used
+        m.reset()
+        assert np.array_equal(m.greedy(5, steps)[0], plain)
+    m.reset()
+    g, pen = so.MinStdRand0(77), so.Penalties(0.8, 0.8, 0.996)
+    tok = 5
+    for i in range(steps):
+        tok = so.sample(pen.apply(m.run(tok)), temperature, top_k, top_p, g)
+        pen.drawn(tok)
+        assert tok == int(toks[i]), i
+    m.close()
+
+
 # ---------------------------------------------------------------------------
 # committed golden vectors (tests/golden/oracle_small_models.npz): the HIP path on the same
 # synthetic models, one-token steps and seq mode, within the stated tolerance of the fixture

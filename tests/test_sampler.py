@@ -110,3 +110,28 @@ def test_empty_logits_raise():
     hs = HostSampler(1)
     with pytest.raises(fr.FrhipError):
         hs.sample(np.zeros(0, np.float32))
+
+
+def test_penalties_of_the_generation_loop_against_their_closed_form():
+    """chat.cpp:57-62, 77: at the draw of step s a token drawn at steps d_1 < d_2 < ... < s has had
+    frequency * sum_j decay^(s - 1 - d_j) + presence subtracted from its logit (each earlier adjustment was made
+    to that step's own logits, not carried over), other tokens nothing.  Checked in float64 against the oracle's
+    fp32 loop for a fixed drawing pattern."""
+    pres, freq, decay = 0.8, 0.8, 0.996
+    pen = so.Penalties(pres, freq, decay)
+    draws = [7, 3, 7, 7, 1, 3, 9, 7, 0, 3, 3, 7]
+    for s, tok in enumerate(draws):
+        logits = np.linspace(-1, 1, 12).astype(np.float32)
+        before = logits.copy()
+        pen.apply(logits)
+        for t in range(12):
+            ds = [d for d in range(s) if draws[d] == t]
+            want = float(before[t]) - (freq * sum(decay ** (s - 1 - d) for d in ds) + pres if ds else 0.0)
+            assert abs(float(logits[t]) - want) <= 1e-5, (s, t)
+        pen.drawn(tok)
+    # decay 1, frequency 1, presence 0: the adjustment is the plain count
+    pen = so.Penalties(0.0, 1.0, 1.0)
+    for tok in (2, 2, 5, 2):
+        pen.drawn(tok)
+    logits = np.zeros(8, np.float32)
+    assert list(pen.apply(logits)) == [0, 0, -3, 0, 0, -1, 0, 0]
