@@ -377,8 +377,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(GemmArgs a) {
 // cycles from barrier to barrier, MFMA waves 1550-1700 plus 540-700 waiting).  In this form a load
 // needs scalar instructions only.  `lds` is the destination's LDS byte address (lane l writes 16 bytes
 // at lds + 16 l); the wait counts are the caller's business, as with the builtin.
+// M0 is written here without the compiler knowing (it refuses m0 in a clobber list: a reserved register).  That is safe
+// as used: a workgroup issues either these loads or the builtin's (a tile lies wholly inside the matrices or it does not),
+// never both, so no value the compiler keeps in M0 for the builtin is ever live across this statement.
 __device__ __forceinline__ void load_lds_saddr(unsigned voff, const void* sbase, unsigned lds) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds) : "memory");
 }
 
 // The same address for every lane, in scalar registers (the compiler cannot always prove it).

@@ -342,16 +342,16 @@ def test_sampled_generation_follows_the_oracle_sampler(model_files):
 
 
 @pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 1, 0.0), (1.2, 50, 0.9)])  # chat.cpp:76-77's own settings; a sampled run
-def test_generation_with_the_repetition_penalties_of_the_chat_loop(model_files, temperature, top_k, top_p):
+def test_generation_with_the_repetition_penalties_of_the_chat_loop(temperature, top_k, top_p):
     """chat.cpp:56-92 with its presence / frequency penalties and their decay (0.8, 0.8, 0.996: chat.cpp:22-24):
     the C++ loop on the hip model draws the tokens that the oracle's sampler draws from the same logits adjusted
-    by the oracle's statement of the penalties, and the penalties change what is drawn."""
+    by the oracle's statement of the penalties, and the penalties change what is drawn (a vocabulary of 64 and 80
+    steps: without penalties some token must repeat, and a repeated token's logit is at least 1.6 lower with them)."""
     import sys
     sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
     import sampler_oracle as so
-    path, params, emb = model_files
-    m = fr.Model(path, "hip fp16")
-    steps = 48
+    m = fr.Model("synthetic:v=4,L=2,C=256,F=1024,V=64,seed=9", "hip fp16")
+    steps = 80
     toks, _ = m.generate(fr.Sampler(77), 5, steps, temperature=temperature, top_k=top_k, top_p=top_p,
                          presence_penalty=0.8, frequency_penalty=0.8, penalty_decay=0.996)
     m.reset()
