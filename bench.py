@@ -219,7 +219,7 @@ def rwkv5_extra(fr):
     m = fr.Model("synthetic:v=5.2,L=32,C=2560,F=8960,V=65536,H=40,seed=1238", "hip int8")
     ids = np.random.default_rng(44).integers(0, V_, 512)
     best = 1e9
-    os.environ["FR_HIP_SEQ_IMAGE"] = "0"  # the uint8 weights expanded to binary16 per call, nothing kept
+    os.environ["FR_HIP_SEQ_IMAGE"] = "0"  # the default: the uint8 weights expanded to binary16 per call, nothing kept
     try:
         for _ in range(3):
             m.reset()
@@ -234,8 +234,8 @@ def rwkv5_extra(fr):
         _, secs = m.greedy(17, 256)
     finally:
         del os.environ["FR_HIP_GREEDY_ON_HOST"]
-    # the same prompt with the binary16 image of the uint8 weights kept on the device (FR_HIP_SEQ_IMAGE=1, the default
-    # on a device of this size: 2 more bytes per weight, no expansion per call); the first pass makes the images and is not timed
+    # the same prompt with the binary16 image of the uint8 weights kept on the device (FR_HIP_SEQ_IMAGE=1, opt-in:
+    # 2 more bytes per weight, no expansion per call); the first pass makes the images and is not timed
     os.environ["FR_HIP_SEQ_IMAGE"] = "1"
     try:
         kept = 1e9

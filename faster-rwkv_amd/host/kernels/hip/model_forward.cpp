@@ -483,7 +483,11 @@ Tensor ModelForwardSeq(Model *model, Device device, const std::vector<int> &ids,
   if (!full_output && ids.size() < 4 && !std::getenv("FR_HIP_SEQ_ALWAYS")) {
     Tensor out;
     for (int id : ids) out = hip::ModelForward(model, device, id);
-    return out;
+    // the one-token result is a view of the plan's pinned ring (valid until the next-but-one call); a prompt's
+    // result belongs to the caller, as the seq operators' does
+    Tensor owned = Tensor::Empty(out.shape(), out.dtype(), Device::kCPU);
+    std::memcpy(owned.data_ptr(), out.data_ptr(), out.nbytes());
+    return owned;
   }
   auto ex = extra_of(model);
   const int T = static_cast<int>(ids.size()), C = model->n_embd();

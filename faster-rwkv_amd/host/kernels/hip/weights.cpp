@@ -51,19 +51,12 @@ const frhip_weight *find_weight(const Tensor &t) {
   return it == table().end() ? nullptr : &it->second->desc;
 }
 
-// FR_HIP_SEQ_IMAGE=1 / 0 decides (read per call, like FR_HIP_GENERIC); unset: kept on a device with 128 GB or more,
-// where the image of even a 14B model (28 GB beside 14 GB of codes) is a small part of the memory.
+// FR_HIP_SEQ_IMAGE=1 keeps the images (read per call, like FR_HIP_GENERIC).  Unset or 0: never -- a caller who chose
+// uint8 weights chose their footprint, and the images would triple it (2 more bytes per weight: a 14B model goes from
+// 14 to 42 GB).  On a 288 GB part that is often the trade to take (no expansion per prompt), so it is one switch away.
 static bool keep_images() {
-  if (const char *e = std::getenv("FR_HIP_SEQ_IMAGE")) return std::atoi(e) != 0;
-  static const bool roomy = [] {
-    (void)stream();  // the device is initialised
-    char name[128];
-    int cus = 0;
-    size_t total = 0;
-    if (frhip_device_info(name, sizeof(name), &cus, &total) != 0) return false;
-    return total >= (static_cast<size_t>(128) << 30);
-  }();
-  return roomy;
+  const char *e = std::getenv("FR_HIP_SEQ_IMAGE");
+  return e != nullptr && std::atoi(e) != 0;
 }
 
 const frhip_weight *find_seq_weight(const Tensor &t, int rows) {

@@ -18,7 +18,8 @@ struct Model {
   // One id -> one-token forward; several -> seq mode.  Logits come back on the CPU (fp32).
   // On the hip device the one-token result is a view of one of two pinned host buffers: it stays
   // valid until the next-but-one Run().  Copy it to keep it longer, or set FR_HIP_OWNED_LOGITS=1
-  // to get a tensor that owns its memory from every call.
+  // to get a tensor that owns its memory from every call.  A prompt (several ids) always returns
+  // a tensor that owns its memory.
   Tensor Run(const std::vector<int> &ids);
   Tensor Run(int id);
   void LoadStateFile(const std::string &path);

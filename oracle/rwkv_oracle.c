@@ -272,15 +272,27 @@ void orc_gemv_u8(const orc_half *x, const uint8_t *q, const orc_half *mx, const 
       c[j] = orc_h2f(rx[n0 + j]) / 255.0f;
       m[j] = orc_h2f(mx[n0 + j]);
     }
-    for (int k = 0; k < K; k++) {
-      const uint8_t *qr = q + (size_t)k * N + n0;
-      const double xk = (double)xf[k];
-      for (int j = 0; j < n1 - n0; j++) {
-        const float a = c[j] * ryf[k];
-        const float b = m[j] + myf[k];
-        const float w32 = fmaf((float)qr[j], a, b);
-        acc[j] += xk * (double)w32;
-        facc[j] += xf[k] * w32; /* ORC_ACC_F32_SEQUENTIAL: fp32 products and sums, ascending k */
+    /* the same weights either way; only the accumulation differs (one loop per mode: the mode is fixed for a call) */
+    if (g_acc_mode == ORC_ACC_F32_SEQUENTIAL) {
+      for (int k = 0; k < K; k++) {
+        const uint8_t *qr = q + (size_t)k * N + n0;
+        for (int j = 0; j < n1 - n0; j++) {
+          const float a = c[j] * ryf[k];
+          const float b = m[j] + myf[k];
+          const float w32 = fmaf((float)qr[j], a, b);
+          facc[j] += xf[k] * w32; /* fp32 products and sums, ascending k */
+        }
+      }
+    } else {
+      for (int k = 0; k < K; k++) {
+        const uint8_t *qr = q + (size_t)k * N + n0;
+        const double xk = (double)xf[k];
+        for (int j = 0; j < n1 - n0; j++) {
+          const float a = c[j] * ryf[k];
+          const float b = m[j] + myf[k];
+          const float w32 = fmaf((float)qr[j], a, b);
+          acc[j] += xk * (double)w32;
+        }
       }
     }
     for (int j = 0; j < n1 - n0; j++)

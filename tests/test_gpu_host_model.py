@@ -129,7 +129,7 @@ def test_seq_mode_equals_one_token_steps_and_oracle(model_files, strategy):
 @pytest.mark.parametrize("spec", ["v=4,L=3,C=512,F=2048,V=2048,seed=11", "v=5.2,L=3,C=512,F=1792,V=2048,H=8,seed=12"])
 @pytest.mark.parametrize("generic", [False, True])
 def test_kept_binary16_image_of_uint8_weights_gives_the_same_bits(spec, generic):
-    """FR_HIP_SEQ_IMAGE=1 (the default on a device with 128 GB or more; =0: off): prompts of
+    """FR_HIP_SEQ_IMAGE=1 (opt-in; unset or 0: off): prompts of
     FRHIP_SEQ_EXPAND_ROWS rows or more multiply the kept binary16 image of the uint8 weights instead
     of one expanded per call; w^ is the same, so logits (last
     row and every row) and the state left behind are the same bits.  One-token steps still read the
@@ -151,7 +151,7 @@ def test_kept_binary16_image_of_uint8_weights_gives_the_same_bits(spec, generic)
     try:
         if generic:
             os.environ["FR_HIP_GENERIC"] = "1"
-        os.environ["FR_HIP_SEQ_IMAGE"] = "0"  # unset it would follow the size of the device's memory
+        os.environ["FR_HIP_SEQ_IMAGE"] = "0"  # the default, stated
         plain = run()
         os.environ.update(env)
         kept = run()
