@@ -601,6 +601,11 @@ struct RowsArgs {
   int prologue;
   int start[kMaxSeg + 1];  // first global row of each segment; start[nseg] = total rows (host bookkeeping)
   int bstart[kMaxSeg + 1]; // first batch of each segment for the launch's R (set at launch)
+  // exclusive != 0: every workgroup serves one segment only (workgroups wg_start[s] .. wg_start[s+1]-1 serve segment s,
+  // whose batches are split over their waves by seg_split[s]); it then loads, stages and sums for that segment alone
+  int exclusive;
+  int wg_start[kMaxSeg + 1];
+  Split seg_split[kMaxSeg];
   Seg seg[kMaxSeg];
   // prologue inputs
   const h1* vec0;                      // P_COPY
@@ -678,7 +683,24 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // The wave index is made visibly uniform: otherwise the lookups in the kernel arguments
   // (segment table, row addresses) become vector loads that every weight load has to wait for.
   int g0, g1;
-  split_even(a.split, grid_wave(a.split), g0, g1);
+  int ws = 0;  // exclusive launches: the one segment this workgroup serves
+  if (a.exclusive) {
+#pragma unroll
+    for (int i = 1; i < kMaxSeg; i++) ws += (i < a.nseg && (int)blockIdx.x >= a.wg_start[i]) ? 1 : 0;
+    const int wgs = a.wg_start[ws + 1] - a.wg_start[ws], lb = (int)blockIdx.x - a.wg_start[ws];
+    const Split sp = a.seg_split[ws];
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // numbered as grid_wave numbers them, within the segment's workgroups
+    split_even(sp, sp.rem != 0 ? wv * wgs + lb : lb * kWaves + wv, g0, g1);
+    g0 += a.bstart[ws];
+    g1 += a.bstart[ws];
+  } else {
+    split_even(a.split, grid_wave(a.split), g0, g1);
+  }
+  // does this workgroup need segment i's operands / staged vector j?
+  auto serves_seg = [&](int i) { return a.exclusive ? i == ws : i < a.nseg; };
+  auto serves_vec = [&](int j) { return a.exclusive ? j == a.seg[ws].vec : j < a.nvec; };
+  const int qmul = a.exclusive ? 0 : 1;  // exclusive: the segment's Sx, Smy are totals 0, 1; else segment s has 2 s, 2 s + 1
 
   struct Meta {
     int seg, loc0, nvalid;  // segment, first row within it, rows of the batch that exist
@@ -752,9 +774,9 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       const int n = m.loc0 + lane;
       if constexpr (U8) {
         // lane v of qtv holds total v of (Sx, Smy) x segments; the segment is uniform here
-        const float q0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums + 0));
-        const float q1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums + 1));
-        mine = finish_q(mine, (float)m.qrx, (float)m.qmx, q0, q1);
+        const float sx_ = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums * qmul + 0));
+        const float smy_ = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qtv), m.seg * kQSums * qmul + 1));
+        mine = finish_q(mine, (float)m.qrx, (float)m.qmx, sx_, smy_);
       }
       run_epilogue(a, sg, n, mine, m.ex, m.er);
     }
@@ -796,12 +818,12 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       sxv = *reinterpret_cast<const h8*>(a.sx + e0);
 #pragma unroll
       for (int i = 0; i < kMaxSeg; i++)
-        if (i < a.nvec) mixv[i] = *reinterpret_cast<const h8*>(a.mix[i] + e0);
+        if (serves_vec(i)) mixv[i] = *reinterpret_cast<const h8*>(a.mix[i] + e0);
     }
     if constexpr (U8) {
 #pragma unroll
       for (int i = 0; i < kMaxSeg; i++)
-        if (i < a.nseg) {
+        if (serves_seg(i)) {
           qry[i] = *reinterpret_cast<const h8*>(a.seg[i].w.ry + e0);
           qmy[i] = *reinterpret_cast<const h8*>(a.seg[i].w.my + e0);
         }
@@ -880,12 +902,12 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
           } else {
 #pragma unroll
             for (int i = 0; i < kMaxSeg; i++)
-              if (i < a.nvec) reinterpret_cast<h8*>(vec_at(i))[threadIdx.x] = mix8(ln.xx, sxv, mixv[i]);
+              if (serves_vec(i)) reinterpret_cast<h8*>(vec_at(i))[threadIdx.x] = mix8(ln.xx, sxv, mixv[i]);
           }
         } else {
 #pragma unroll
           for (int i = 0; i < kMaxSeg; i++) {
-            if (i < a.nseg) {
+            if (serves_seg(i)) {
               h8 x = ln.xx;
               if constexpr (PRO == P_LN_MIX) {
                 // segment i multiplies staged vector seg[i].vec; pick its mix without dynamic register indexing
@@ -903,9 +925,10 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
         if (PRO == P_LN_MIX && blockIdx.x == 0) *reinterpret_cast<h8*>(a.xx_out + e0) = ln.xx;
       }
     }
-    for (int i = 0; i < (U8 ? a.nseg : a.nvec); i++) zero_pad<U8>(vec_at(i), nchunk, kPad);
+    for (int i = 0; i < (U8 ? a.nseg : a.nvec); i++)
+      if (U8 ? serves_seg(i) : serves_vec(i)) zero_pad<U8>(vec_at(i), nchunk, kPad);
     // (a ready vector is staged within a fraction of a microsecond and its rows are few: there the sums stay ahead of the barrier)
-    if constexpr (U8 && PRO == P_COPY) publish_qsums(part, a.nseg * kQSums, qred);
+    if constexpr (U8 && PRO == P_COPY) publish_qsums(part, a.nseg * kQSums, qred);  // (one segment: never exclusive)
     __syncthreads();
   }
   // ---- the rest of the first batch ----
@@ -919,11 +942,16 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     if constexpr (PRO != P_COPY) {
 #pragma unroll
       for (int i = 0; i < kMaxSeg; i++)
-        if (i < a.nseg) sum_q(qx[i], qmy[i], part + i * kQSums);
-      publish_qsums(part, a.nseg * kQSums, qred);
+        if (serves_seg(i)) {
+          if (a.exclusive)
+            sum_q(qx[i], qmy[i], part);
+          else
+            sum_q(qx[i], qmy[i], part + i * kQSums);
+        }
+      publish_qsums(part, (a.exclusive ? 1 : a.nseg) * kQSums, qred);
       __syncthreads();
     }
-    qtv = gather_qsums(a.nseg * kQSums, qred);
+    qtv = gather_qsums((a.exclusive ? 1 : a.nseg) * kQSums, qred);
   }
 
   if constexpr (!MULTI) {
@@ -1336,6 +1364,47 @@ static long count_batches(const RowsArgs& a, int R) {
   return nb;
 }
 
+// Workgroups per segment for a launch whose workgroups serve one segment each: in proportion to the segments'
+// batches, at least one each, summing to the grid.  Returns false when the grid has fewer workgroups than segments.
+static bool share_workgroups(const RowsArgs& a, int R, int grid, int (&wgs)[kMaxSeg]) {
+  if (grid < a.nseg) return false;
+  long nb[kMaxSeg], total = 0;
+  for (int s = 0; s < a.nseg; s++) {
+    nb[s] = (a.seg[s].w.N + R - 1) / R;
+    total += nb[s];
+  }
+  int given = 0, widest = 0;
+  for (int s = 0; s < a.nseg; s++) {
+    wgs[s] = (int)((nb[s] * grid + total / 2) / total);
+    if (wgs[s] < 1) wgs[s] = 1;
+    given += wgs[s];
+    if (nb[s] > nb[widest]) widest = s;
+  }
+  wgs[widest] += grid - given;  // rounding: the segment with the most batches takes the difference
+  return wgs[widest] >= 1;
+}
+
+// Every segment's batches fit one per wave of its own workgroups?
+static bool exclusive_fits(const RowsArgs& a, int R, int grid) {
+  int wgs[kMaxSeg];
+  if (!share_workgroups(a, R, grid, wgs)) return false;
+  for (int s = 0; s < a.nseg; s++)
+    if ((long)(a.seg[s].w.N + R - 1) / R > (long)wgs[s] * kWaves) return false;
+  return true;
+}
+
+// A launch of several matrices after a layernorm can give every workgroup one matrix only: the workgroup then loads and
+// stages one mixed vector (uint8: one set of ry / my, two sums) instead of all of them.  FRHIP_SEG_EXCLUSIVE=0: off.
+// Measured (decode tok/s, exclusive against shared): RWKV-5.2 3B uint8 845 against 772, RWKV-4 1.5B uint8 1635 against 1594,
+// RWKV-5.2 3B binary16 (four matrices) 741 against 736; binary16 launches of two matrices lose half a percent (1419
+// against 1426: their workgroups stage two 4 KB vectors either way), so those stay shared.  FRHIP_SEG_EXCLUSIVE=0 / 1
+// forces it off / on for every such launch.
+static bool want_exclusive(const RowsArgs& a, bool u8) {
+  static const int forced = getenv("FRHIP_SEG_EXCLUSIVE") ? atoi(getenv("FRHIP_SEG_EXCLUSIVE")) : -1;
+  if (a.nseg < 2 || a.prologue != P_LN_MIX || forced == 0) return false;
+  return forced > 0 || u8 || a.nseg >= 3;
+}
+
 static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
   static const int max_u8 = env_int("FRHIP_MAXLOADS_U8", kMaxLoads);
   const int kMaxLoads = u8 ? max_u8 : frhip::kMaxLoads;
@@ -1345,7 +1414,7 @@ static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
   if (rmax > 6) rmax = 6;
   // the smallest R for which every wave gets at most one batch: a single register-resident batch
   for (int r = 1; r <= rmax; r++)
-    if (count_batches(a, r) <= waves) {
+    if (want_exclusive(a, u8) ? exclusive_fits(a, r, grid) : count_batches(a, r) <= waves) {
       *multi = false;
       return r;
     }
@@ -1511,6 +1580,16 @@ static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char
   for (int s = 0; s < kMaxSeg; s++)
     a.bstart[s + 1] = s < a.nseg ? a.bstart[s] + (a.seg[s].w.N + R - 1) / R : INT_MAX;
   a.split = make_split(a.bstart[a.nseg], grid);
+  a.exclusive = 0;
+  int wgs[kMaxSeg];
+  if (want_exclusive(a, u8) && share_workgroups(a, R, grid, wgs)) {
+    a.exclusive = 1;
+    a.wg_start[0] = 0;
+    for (int s = 0; s < kMaxSeg; s++) {
+      a.wg_start[s + 1] = s < a.nseg ? a.wg_start[s] + wgs[s] : INT_MAX;
+      if (s < a.nseg) a.seg_split[s] = make_split(a.bstart[s + 1] - a.bstart[s], wgs[s]);
+    }
+  }
   const size_t lds = staged_bytes(nch, u8) * (u8 ? a.nseg : a.nvec);
   FR_TRY(check_lds(lds));
   bool ok = false;
