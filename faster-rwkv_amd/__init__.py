@@ -97,6 +97,7 @@ _SIGS = {
     "frhip_att_one_v5": (_i, [_i, _i] + [_vp] * 12 + [_WP] * 4 + [_vp] * 5),
     "frhip_argmax_f32": (_i, [_vp, _i, _vp, _vp]),
     "frhip_argmax_blocks_f32": (_i, [_vp, _i, _vp, _i, _vp]),
+    "frhip_argmax_blocks_f32_mirror": (_i, [_vp, _i, _vp, _vp, _i, _vp]),
     "frhip_gemm": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
     "frhip_gemm_act": (_i, [_vp, _WP, _vp, _i, _i, _vp]),
     "frhip_copy_probe": (_i, [_vp, _vp, _sz, _vp]),

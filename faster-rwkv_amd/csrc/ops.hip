@@ -260,7 +260,7 @@ __global__ __launch_bounds__(512) void read_probe_kernel(const u32x4* __restrict
 // empty: it reports -inf at index n).  The caller reduces the pairs (greater value, then smaller
 // index): with the logits in one slab that is 64 pairs instead of 65 536 values.
 __global__ __launch_bounds__(256) void argmax_blocks_f32_kernel(const float* __restrict__ x, int n, int len,
-                                                              float* pairs) {
+                                                              float* pairs, float* mirror) {
   __shared__ float bv[4];
   __shared__ int bi[4];
   const int lo = blockIdx.x * len;
@@ -301,6 +301,10 @@ __global__ __launch_bounds__(256) void argmax_blocks_f32_kernel(const float* __r
       }
     pairs[2 * blockIdx.x] = best;
     reinterpret_cast<int32_t*>(pairs)[2 * blockIdx.x + 1] = idx;
+    if (mirror) {  // a second copy, e.g. in pinned host memory beside the logits
+      mirror[2 * blockIdx.x] = best;
+      reinterpret_cast<int32_t*>(mirror)[2 * blockIdx.x + 1] = idx;
+    }
   }
 }
 
@@ -654,14 +658,18 @@ int frhip_read_probe(const void* src, size_t bytes, void* sink, frhip_stream s) 
   return check_launch("read_probe");
 }
 
-int frhip_argmax_blocks_f32(const float* x, int n, void* pairs, int nblocks, frhip_stream s) {
+int frhip_argmax_blocks_f32_mirror(const float* x, int n, void* pairs, void* mirror, int nblocks, frhip_stream s) {
   if (!x || !pairs) return set_error(FRHIP_EINVAL, "argmax: null pointer");
   if (n <= 0 || nblocks <= 0) return set_error(FRHIP_ESHAPE, "argmax: empty input");
   if (reinterpret_cast<uintptr_t>(x) % 16) return set_error(FRHIP_EINVAL, "argmax: x must be 16-byte aligned");
   const int len = ((n + nblocks - 1) / nblocks + 3) / 4 * 4;
   hipLaunchKernelGGL(argmax_blocks_f32_kernel, dim3(nblocks), dim3(256), 0, static_cast<hipStream_t>(s), x, n, len,
-                     static_cast<float*>(pairs));
+                     static_cast<float*>(pairs), static_cast<float*>(mirror));
   return check_launch("argmax_blocks");
+}
+
+int frhip_argmax_blocks_f32(const float* x, int n, void* pairs, int nblocks, frhip_stream s) {
+  return frhip_argmax_blocks_f32_mirror(x, n, pairs, nullptr, nblocks, s);
 }
 
 int frhip_argmax_f32(const float* logits, int n, int32_t* out_id, frhip_stream s) {

@@ -37,6 +37,7 @@ struct DecodePlan {
   int L = 0, C = 0, F = 0, V = 0, n_logits = 0;
   Tensor x, ws, counter;
   Tensor logits_dev;
+  Tensor pairs_dev[2];                         // the arg-max pairs of the step on parity 0 / 1, for the device-side greedy loop
   float *logits_host[2] = {nullptr, nullptr};  // pinned; the head kernel stores the logits here too, the arg-max pairs follow
   int32_t *ring = nullptr;                     // pinned; token ids, read by the first kernel
   uint32_t fed = 0;                            // tokens fed so far == the device counter
@@ -114,6 +115,10 @@ static std::shared_ptr<DecodePlan> make_plan(Model *model, ModelExtra &ex) {
   FRHIP_CHECK(frhip_fill(p->counter.data_ptr(), FRHIP_F32, 0.0f, 1, stream()));  // all-zero bits
   p->n_logits = static_cast<int>(model->_params.back().size(1));
   p->logits_dev = Tensor::Empty({p->n_logits}, DType::kFloat32, d);
+  for (auto &pd : p->pairs_dev) {
+    pd = Tensor::Empty({2 * DecodePlan::kArgmaxBlocks}, DType::kFloat32, d);
+    FRHIP_CHECK(frhip_fill(pd.data_ptr(), FRHIP_F32, 0.0f, 2 * DecodePlan::kArgmaxBlocks, stream()));
+  }
   void *h = nullptr;
   FRHIP_CHECK(frhip_host_malloc(&h, sizeof(int32_t) * DecodePlan::kRing));
   p->ring = static_cast<int32_t *>(h);
@@ -192,7 +197,7 @@ static void adopt_states(Model *model, DecodePlan &p) {
   }
 }
 
-// `chained`: the token comes from the arg-max pairs the previous step left behind its logits
+// `chained`: the token comes from the arg-max pairs the previous step left in device memory (pairs_dev)
 // (that step ran on the other parity) instead of from the host's ring.
 static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chained = false) {
   const auto &P = model->_params;
@@ -200,7 +205,7 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chaine
   const int C = p.C, F = p.F;
   const int cur = p.parity, nxt = 1 - p.parity;
   if (chained)
-    FRHIP_CHECK(frhip_embed_argmax(ex.emb_table.data_ptr(), p.V, 2 * C, p.logits_host[nxt] + p.n_logits,
+    FRHIP_CHECK(frhip_embed_argmax(ex.emb_table.data_ptr(), p.V, 2 * C, p.pairs_dev[nxt].data_ptr(),
                                    DecodePlan::kArgmaxBlocks, p.chain_ids, DecodePlan::kChainIds,
                                    reinterpret_cast<uint32_t *>(p.counter.data_ptr()), p.x.data_ptr(), s));
   else
@@ -272,8 +277,9 @@ static void issue_token(Model *model, ModelExtra &ex, DecodePlan &p, bool chaine
   // A caller that only wants the most likely token need not read 4 * V bytes of fresh host memory.
   FRHIP_CHECK(frhip_head_mirror(C, p.x.data_ptr(), P[pi].data_ptr(), P[pi + 1].data_ptr(), hw,
                                 p.logits_dev.data_ptr<float>(), p.logits_host[cur], s));
-  FRHIP_CHECK(frhip_argmax_blocks_f32(p.logits_dev.data_ptr<float>(), p.n_logits, p.logits_host[cur] + p.n_logits,
-                                      DecodePlan::kArgmaxBlocks, s));
+  // the pairs twice: in device memory for a next step that picks its own token, beside the host's logits for the host
+  FRHIP_CHECK(frhip_argmax_blocks_f32_mirror(p.logits_dev.data_ptr<float>(), p.n_logits, p.pairs_dev[cur].data_ptr(),
+                                             p.logits_host[cur] + p.n_logits, DecodePlan::kArgmaxBlocks, s));
 }
 
 // Captures `count` consecutive tokens, the first on parity `parity`, as one graph; nothing runs, and the

@@ -311,6 +311,10 @@ int frhip_argmax_f32(const float *logits, int n, int32_t *out_id, frhip_stream s
  * bytes; an empty slice reports -inf at index n); the second step, over the pairs (greater value,
  * then smaller index), is the caller's. */
 int frhip_argmax_blocks_f32(const float *x, int n, void *pairs, int nblocks, frhip_stream s);
+/* The same with the pairs stored twice: to `pairs` and, if not NULL, to `mirror` (e.g. `pairs` in device memory
+ * for a next step that picks its token on the device, `mirror` in pinned host memory beside the logits the host
+ * reads, chat.cpp:76-87). */
+int frhip_argmax_blocks_f32_mirror(const float *x, int n, void *pairs, void *mirror, int nblocks, frhip_stream s);
 
 #ifdef __cplusplus
 }

@@ -193,6 +193,10 @@ def test_argmax_blocks_first_of_ties(n, nblocks):
     pairs = DevBuf.empty(2 * nblocks, np.float32)
     fr.check(L().frhip_argmax_blocks_f32(keep(x).ptr, n, pairs.ptr, nblocks, None))
     raw = pairs.numpy()
+    # the two-destination form stores the same pairs twice
+    first, second = DevBuf.empty(2 * nblocks, np.float32), DevBuf.empty(2 * nblocks, np.float32)
+    fr.check(L().frhip_argmax_blocks_f32_mirror(keep(x).ptr, n, first.ptr, second.ptr, nblocks, None))
+    assert first.numpy().tobytes() == raw.tobytes() == second.numpy().tobytes()
     vals, idxs = raw[0::2], raw[1::2].view(np.int32)
     best, at = -np.inf, n
     for v, i in zip(vals, idxs):
