@@ -17,7 +17,8 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-LIBFRHIP = os.path.join(HERE, "libfrhip.so")
+# FRHIP_LIBRARY: another build of the same library (the measurement build libfrhip_timeline.so, see timeline.py)
+LIBFRHIP = os.environ.get("FRHIP_LIBRARY") or os.path.join(HERE, "libfrhip.so")
 LIBHOST = os.path.join(HERE, "libfr_host.so")
 
 F32, F16, U8 = 0, 1, 2

@@ -37,6 +37,37 @@ namespace frhip {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / kWave;
+
+// Measurement build (`make timeline` -> -DFRHIP_TIMELINE, a library of its own): every wave of rows_kernel notes the
+// 100 MHz clock at the points marked FR_TL(i), keeps the notes in registers and leaves them in g_timeline[slot][wave]
+// when it ends (so the notes add no memory operation before the kernel's last store); launches take the slots round
+// robin; frhip_timeline_read copies them out.  Compiled out otherwise.
+#ifdef FRHIP_TIMELINE
+constexpr int kTlStamps = 16, kTlSlots = 8, kTlWaves = 4096;
+__device__ unsigned long long g_timeline[kTlSlots][kTlWaves][kTlStamps];
+static int g_timeline_launches = 0;
+#define FR_TL_DECL unsigned long long fr_tl[kTlStamps] = {}
+#define FR_TL(i) fr_tl[i] = __builtin_amdgcn_s_memrealtime()
+#define FR_TL_AFTER(i, v)            \
+  do {                               \
+    asm volatile("" ::"v"(v));       \
+    FR_TL(i);                        \
+  } while (0)
+#define FR_TL_FLUSH(slot)                                                                            \
+  do {                                                                                               \
+    __builtin_amdgcn_s_waitcnt(0);                                                                   \
+    FR_TL(kTlStamps - 1);                                                                            \
+    const int fr_w = (int)blockIdx.x * kWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave); \
+    if ((threadIdx.x & (kWave - 1)) == 0 && fr_w < kTlWaves) {                                       \
+      for (int fr_i = 0; fr_i < kTlStamps; fr_i++) g_timeline[slot][fr_w][fr_i] = fr_tl[fr_i];      \
+    }                                                                                                \
+  } while (0)
+#else
+#define FR_TL_DECL
+#define FR_TL(i)
+#define FR_TL_AFTER(i, v)
+#define FR_TL_FLUSH(slot)
+#endif
 constexpr int kMaxSeg = 4;
 constexpr int kFusedMaxC = 8 * kThreads;  // widest vector the fused layernorm prologues take
 constexpr int kMaxC = 16384;
@@ -618,6 +649,9 @@ struct RowsArgs {
   int res_n;        // elements of res_x / res_r that may be read (1 when no epilogue uses them)
   float* mirror;    // E_LOGITS: second destination of every value (memory the host reads), or null
   int div2;
+#ifdef FRHIP_TIMELINE
+  int tl_slot;  // where the launch leaves its timestamps
+#endif
 };
 
 __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, int n, float sum, h1 ex, h1 er) {
@@ -662,6 +696,8 @@ template <int R, int NCH, bool U8, bool MULTI, int PRO>
 __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float red[2 * kWaves];
+  FR_TL_DECL;
+  FR_TL(0);  // entry
   // One field from every 64-byte line of the kernel arguments is requested up front, so that the
   // scalar loads further down (issued where each field is first needed) hit the scalar cache.
   asm volatile("" ::"s"(a.K), "s"(a.seg[0].out), "s"(a.seg[1].out), "s"(a.seg[2].out), "s"(a.seg[3].out), "s"(a.vec0),
@@ -764,12 +800,14 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     const Seg& sg = a.seg[m.seg];
     float acc[R];
     b.dot_shared(vec_at(U8 ? m.seg : sg.vec), lane, acc);
+    FR_TL_AFTER(8, acc[0]);  // products done (of the wave's last batch)
     float mine = 0.f;
 #pragma unroll
     for (int r = 0; r < R; r++) {
       const float t = wave_sum(acc[r]);
       if (lane == r) mine = t;
     }
+    FR_TL_AFTER(9, mine);  // reduced
     if (lane < m.nvalid) {
       const int n = m.loc0 + lane;
       if constexpr (U8) {
@@ -792,21 +830,34 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // thread; P_LN / P_LN_MIX: K <= 8 * kThreads, one group per thread.  Only threads that own a
   // group load (every byte requested here passes through the compute unit's vector memory
   // pipeline ahead of the rows): branches are harmless before the rows, whose count is fixed.
-  constexpr int kCopyPasses = (NCH * kWave * (U8 ? 2 : 1) + kThreads - 1) / kThreads;
+  // P_COPY, uint8 (three operand vectors: the vector, ry, my): the first four waves of the workgroup (one per SIMD, the
+  // ones the compute unit serves first) load and stage all of them, so the pieces are at the head of the compute unit's
+  // queue (data returns in request order across the waves: an operand requested by wave 7 behind the rows of waves 0-6
+  // arrives after them).  Where a batch is more than 8 loads the rows of those four waves alone fill what a compute unit
+  // keeps in flight (about 64 KB) and the other four would be held at their load instructions, and with them the barrier
+  // that releases the staged vector: there they go to the barrier first and request their rows behind it.
+  // Measured (decode tok/s, one box, alternating): RWKV-4 1.5B uint8 1 634 -> 1 644, RWKV-5.2 3B uint8 845 -> 851; the same
+  // for binary16 (one operand vector) 1 430 -> 1 424 and 746 -> 740, so binary16 keeps every thread loading its own group.
+  constexpr bool kStagerMode = PRO == P_COPY && U8;
+  constexpr int kStageWaves = kStagerMode ? 4 : kWaves, kStageThreads = kStageWaves * kWave;
+  constexpr int kCopyPasses = (NCH * kWave * (U8 ? 2 : 1) + kStageThreads - 1) / kStageThreads;
+  const bool stager = (int)threadIdx.x < kStageThreads;  // uniform within a wave
   const int ngrp = K >> 3;
   const bool own = (int)threadIdx.x < ngrp;
   const int e0 = threadIdx.x * 8;
   h8 cx[kCopyPasses] = {}, cry[kCopyPasses] = {}, cmy[kCopyPasses] = {};
   h8 xv{}, lg{}, lb{}, sxv{}, mixv[kMaxSeg] = {}, qry[kMaxSeg] = {}, qmy[kMaxSeg] = {};
   if constexpr (PRO == P_COPY) {
+    if (stager) {
 #pragma unroll
-    for (int p = 0; p < kCopyPasses; p++) {
-      const int g = (int)threadIdx.x + p * kThreads;
-      if (g < ngrp) {
-        cx[p] = reinterpret_cast<const h8*>(a.vec0)[g];
-        if constexpr (U8) {
-          cry[p] = reinterpret_cast<const h8*>(a.seg[0].w.ry)[g];
-          cmy[p] = reinterpret_cast<const h8*>(a.seg[0].w.my)[g];
+      for (int p = 0; p < kCopyPasses; p++) {
+        const int g = (int)threadIdx.x + p * kStageThreads;
+        if (g < ngrp) {
+          cx[p] = reinterpret_cast<const h8*>(a.vec0)[g];
+          if constexpr (U8) {
+            cry[p] = reinterpret_cast<const h8*>(a.seg[0].w.ry)[g];
+            cmy[p] = reinterpret_cast<const h8*>(a.seg[0].w.my)[g];
+          }
         }
       }
     }
@@ -830,10 +881,20 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     }
   }
 
+  FR_TL(1);  // the prologue's operands requested
   // ---- first batch of rows: the chunks that go out ahead of the prologue (see RowBatch::kHead) ----
   RowBatch<R, NCH, U8> A;
-  request_rows(A, whA, J0{}, JH{});
-  if constexpr (!U8) request_ops(mA);
+  constexpr bool kAllRowsFirst = R * NCH <= 8;
+  if constexpr (kStagerMode) {
+    if (kAllRowsFirst || stager) {
+      request_rows(A, whA, J0{}, JN{});
+      request_ops(mA);
+    }
+  } else {
+    request_rows(A, whA, J0{}, JH{});
+    if constexpr (!U8) request_ops(mA);
+  }
+  FR_TL(2);  // first rows requested
 
   // ---- prologue: stage the activation vector(s) in LDS ----
   // uint8: Sx and Smy of every staged vector are needed only when a row is finished.  They are summed behind the
@@ -845,14 +906,16 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   h8 qx[kMaxSeg] = {};
   {
     if constexpr (PRO == P_COPY) {
+      if (stager) {
 #pragma unroll
-      for (int p = 0; p < kCopyPasses; p++) {
-        const int g = (int)threadIdx.x + p * kThreads;
-        if (g < ngrp) {
-          if constexpr (!U8)
-            reinterpret_cast<h8*>(vec_at(0))[g] = cx[p];
-          else
-            stage_q(reinterpret_cast<float*>(vec_at(0)), g, kPad, cx[p], cry[p], cmy[p], part);
+        for (int p = 0; p < kCopyPasses; p++) {
+          const int g = (int)threadIdx.x + p * kStageThreads;
+          if (g < ngrp) {
+            if constexpr (!U8)
+              reinterpret_cast<h8*>(vec_at(0))[g] = cx[p];
+            else
+              stage_q(reinterpret_cast<float*>(vec_at(0)), g, kPad, cx[p], cry[p], cmy[p], part);
+          }
         }
       }
     } else if (PRO == P_LN && K > kFusedMaxC) {
@@ -895,6 +958,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       }
     } else {
       LnOut ln = ln_regs(xv, lg, lb, own, K, red);
+      FR_TL_AFTER(3, (float)ln.xx[0]);  // normalised (the vector has arrived, both reductions are through)
       if (ln.active) {
         if constexpr (!U8) {
           if constexpr (PRO == P_LN) {
@@ -929,14 +993,23 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       if (U8 ? serves_seg(i) : serves_vec(i)) zero_pad<U8>(vec_at(i), nchunk, kPad);
     // (a ready vector is staged within a fraction of a microsecond and its rows are few: there the sums stay ahead of the barrier)
     if constexpr (U8 && PRO == P_COPY) publish_qsums(part, a.nseg * kQSums, qred);  // (one segment: never exclusive)
+    FR_TL(4);  // staged: at the barrier
     __syncthreads();
+    FR_TL(5);  // through the barrier
   }
   // ---- the rest of the first batch ----
-  request_rows(A, whA, JH{}, JN{});
-  // uint8: the per-row operands (two more 2-byte loads per lane: rx, mx) go out behind all rows of the batch; ahead of
-  // the prologue they cost these launches more than the memory latency they save at the end (decode kernels 0.588 ->
-  // 0.583 ms per token; binary16, with at most two such loads, the other way round: 0.662 -> 0.669).
-  if constexpr (U8) request_ops(mA);
+  if constexpr (kStagerMode) {
+    if (!kAllRowsFirst && !stager) {
+      request_rows(A, whA, J0{}, JN{});
+      request_ops(mA);
+    }
+  } else {
+    request_rows(A, whA, JH{}, JN{});
+    // uint8: the per-row operands (two more 2-byte loads per lane: rx, mx) go out behind all rows of the batch; ahead of
+    // the prologue they cost these launches more than the memory latency they save at the end (decode kernels 0.588 ->
+    // 0.583 ms per token; binary16, with at most two such loads, the other way round: 0.662 -> 0.669).
+    if constexpr (U8) request_ops(mA);
+  }
   if constexpr (U8) {
     // (every thread reaches the second barrier; threads without a group add zeros; the wide layernorm has summed already)
     if constexpr (PRO != P_COPY) {
@@ -953,6 +1026,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     }
     qtv = gather_qsums((a.exclusive ? 1 : a.nseg) * kQSums, qred);
   }
+  FR_TL_AFTER(6, qtv);  // all rows of the first batch requested (uint8: Sx, Smy gathered)
 
   if constexpr (!MULTI) {
     consume(A, mA);  // the host guarantees at most one batch per wave
@@ -981,6 +1055,8 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
       }
     }
   }
+  FR_TL(10);  // epilogue issued
+  FR_TL_FLUSH(a.tl_slot);  // waits for the wave's stores, notes the time, writes the notes
 }
 
 // ===========================================================================
@@ -1592,6 +1668,9 @@ static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char
   }
   const size_t lds = staged_bytes(nch, u8) * (u8 ? a.nseg : a.nvec);
   FR_TRY(check_lds(lds));
+#ifdef FRHIP_TIMELINE
+  a.tl_slot = (g_timeline_launches++) % kTlSlots;
+#endif
   bool ok = false;
   switch (nch) {
     case 1: ok = launch_rows_n<1>(R, u8, multi, grid, lds, st, a); break;
@@ -2034,3 +2113,13 @@ extern "C" int frhip_gemv(const void* x, const frhip_weight* w, void* y, int out
   add_seg(a, w, 0, out_dtype == FRHIP_F32 ? E_STORE_F32 : E_STORE_F16, y);
   return launch_rows(a, w->dtype == FRHIP_U8, static_cast<hipStream_t>(s), "gemv");
 }
+
+#ifdef FRHIP_TIMELINE
+// Measurement build only: copies the timestamps of the last 8 row-kernel launches to `dst`
+// ([8 slots][4096 waves][16] uint64, 100 MHz ticks; launch number n took slot n % 8) and reports how many
+// launches have taken a slot so far.
+extern "C" int frhip_timeline_read(void* dst, int* launches) {
+  *launches = frhip::g_timeline_launches;
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(frhip::g_timeline), sizeof(frhip::g_timeline));
+}
+#endif
