@@ -632,11 +632,6 @@ struct RowsArgs {
   int prologue;
   int start[kMaxSeg + 1];  // first global row of each segment; start[nseg] = total rows (host bookkeeping)
   int bstart[kMaxSeg + 1]; // first batch of each segment for the launch's R (set at launch)
-  // exclusive != 0: every workgroup serves one segment only (workgroups wg_start[s] .. wg_start[s+1]-1 serve segment s,
-  // whose batches are split over their waves by seg_split[s]); it then loads, stages and sums for that segment alone
-  int exclusive;
-  int wg_start[kMaxSeg + 1];
-  Split seg_split[kMaxSeg];
   Seg seg[kMaxSeg];
   // prologue inputs
   const h1* vec0;                      // P_COPY
@@ -653,6 +648,16 @@ struct RowsArgs {
   int tl_slot;  // where the launch leaves its timestamps
 #endif
 };
+
+// Every workgroup serves one segment only: workgroups wg_start[s] .. wg_start[s+1]-1 serve segment s, whose batches are
+// split over their waves by seg_split[s]; the workgroup then loads, stages and sums for that segment alone.  A second
+// kernel argument of the launches of that form only: the arguments of the shared form stay as long as they were (56
+// bytes of padding at their end, read by nobody, took 0.7-1.4 % off the decode rate of every model measured).
+struct ExclArgs {
+  int wg_start[kMaxSeg + 1];
+  Split seg_split[kMaxSeg];
+};
+struct NoExclArgs {};
 
 __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, int n, float sum, h1 ex, h1 er) {
   switch (sg.epi) {
@@ -692,8 +697,11 @@ __device__ __forceinline__ void run_epilogue(const RowsArgs& a, const Seg& sg, i
 // issued, so the prologue runs while the rows are in flight and the products start on the
 // first chunks that arrive; a load inside a branch would make the number of loads in flight
 // path-dependent and turn every later wait into a wait for all of them.
-template <int R, int NCH, bool U8, bool MULTI, int PRO>
-__global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
+// EXCL: every workgroup serves one segment only (RowsArgs::exclusive); a parameter of the kernel, not a field it tests,
+// because the test and the lookups behind it cost every launch of the shared form 1.5-2 % (decode tok/s with and
+// without the branch in the code: 1 428 against 1 449 binary16, 746 against 761 for the 3B RWKV-5.2).
+template <int R, int NCH, bool U8, bool MULTI, int PRO, bool EXCL, class XA>
+__device__ __forceinline__ void rows_body(const RowsArgs& a, const XA& xa) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float red[2 * kWaves];
   FR_TL_DECL;
@@ -702,6 +710,13 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // scalar loads further down (issued where each field is first needed) hit the scalar cache.
   asm volatile("" ::"s"(a.K), "s"(a.seg[0].out), "s"(a.seg[1].out), "s"(a.seg[2].out), "s"(a.seg[3].out), "s"(a.vec0),
                "s"(a.res_x));
+  static_assert(offsetof(RowsArgs, seg[0].out) / 64 == 1 && offsetof(RowsArgs, seg[1].out) / 64 == 2 &&
+                    offsetof(RowsArgs, seg[2].out) / 64 == 3 && offsetof(RowsArgs, seg[3].out) / 64 == 4 &&
+                    offsetof(RowsArgs, vec0) / 64 == 5 && offsetof(RowsArgs, mix[2]) / 64 == 5 &&
+                    offsetof(RowsArgs, mix[3]) / 64 == 6 && offsetof(RowsArgs, res_x) / 64 == 6 &&
+                    offsetof(RowsArgs, div2) / 64 == 6,
+                "the list above must name one field of every 64-byte line of the arguments the shared form reads");
+  if constexpr (EXCL) asm volatile("" ::"s"(xa.wg_start[1]), "s"(xa.seg_split[3].rem));
   const int K = a.K;
   const int nchunk = U8 ? (K >> 4) : (K >> 3);
   const size_t row_bytes = U8 ? (size_t)K : 2 * (size_t)K;
@@ -720,11 +735,11 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   // (segment table, row addresses) become vector loads that every weight load has to wait for.
   int g0, g1;
   int ws = 0;  // exclusive launches: the one segment this workgroup serves
-  if (a.exclusive) {
+  if constexpr (EXCL) {
 #pragma unroll
-    for (int i = 1; i < kMaxSeg; i++) ws += (i < a.nseg && (int)blockIdx.x >= a.wg_start[i]) ? 1 : 0;
-    const int wgs = a.wg_start[ws + 1] - a.wg_start[ws], lb = (int)blockIdx.x - a.wg_start[ws];
-    const Split sp = a.seg_split[ws];
+    for (int i = 1; i < kMaxSeg; i++) ws += (i < a.nseg && (int)blockIdx.x >= xa.wg_start[i]) ? 1 : 0;
+    const int wgs = xa.wg_start[ws + 1] - xa.wg_start[ws], lb = (int)blockIdx.x - xa.wg_start[ws];
+    const Split sp = xa.seg_split[ws];
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     // numbered as grid_wave numbers them, within the segment's workgroups
     split_even(sp, sp.rem != 0 ? wv * wgs + lb : lb * kWaves + wv, g0, g1);
@@ -734,9 +749,9 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
     split_even(a.split, grid_wave(a.split), g0, g1);
   }
   // does this workgroup need segment i's operands / staged vector j?
-  auto serves_seg = [&](int i) { return a.exclusive ? i == ws : i < a.nseg; };
-  auto serves_vec = [&](int j) { return a.exclusive ? j == a.seg[ws].vec : j < a.nvec; };
-  const int qmul = a.exclusive ? 0 : 1;  // exclusive: the segment's Sx, Smy are totals 0, 1; else segment s has 2 s, 2 s + 1
+  auto serves_seg = [&](int i) { return EXCL ? i == ws : i < a.nseg; };
+  auto serves_vec = [&](int j) { return EXCL ? j == a.seg[ws].vec : j < a.nvec; };
+  const int qmul = EXCL ? 0 : 1;  // exclusive: the segment's Sx, Smy are totals 0, 1; else segment s has 2 s, 2 s + 1
 
   struct Meta {
     int seg, loc0, nvalid;  // segment, first row within it, rows of the batch that exist
@@ -1016,15 +1031,15 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
 #pragma unroll
       for (int i = 0; i < kMaxSeg; i++)
         if (serves_seg(i)) {
-          if (a.exclusive)
+          if (EXCL)
             sum_q(qx[i], qmy[i], part);
           else
             sum_q(qx[i], qmy[i], part + i * kQSums);
         }
-      publish_qsums(part, (a.exclusive ? 1 : a.nseg) * kQSums, qred);
+      publish_qsums(part, (EXCL ? 1 : a.nseg) * kQSums, qred);
       __syncthreads();
     }
-    qtv = gather_qsums((a.exclusive ? 1 : a.nseg) * kQSums, qred);
+    qtv = gather_qsums((EXCL ? 1 : a.nseg) * kQSums, qred);
   }
   FR_TL_AFTER(6, qtv);  // all rows of the first batch requested (uint8: Sx, Smy gathered)
 
@@ -1057,6 +1072,17 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
   }
   FR_TL(10);  // epilogue issued
   FR_TL_FLUSH(a.tl_slot);  // waits for the wave's stores, notes the time, writes the notes
+}
+
+template <int R, int NCH, bool U8, bool MULTI, int PRO>
+__global__ __launch_bounds__(kThreads) void rows_kernel(RowsArgs a) {
+  rows_body<R, NCH, U8, MULTI, PRO, false>(a, NoExclArgs{});
+}
+
+// The form in which every workgroup serves one segment (layernorm + mix launches of several matrices only).
+template <int R, int NCH, bool U8, bool MULTI>
+__global__ __launch_bounds__(kThreads) void rows_excl_kernel(RowsArgs a, ExclArgs xa) {
+  rows_body<R, NCH, U8, MULTI, P_LN_MIX, true>(a, xa);
 }
 
 // ===========================================================================
@@ -1470,15 +1496,16 @@ static bool exclusive_fits(const RowsArgs& a, int R, int grid) {
 }
 
 // A launch of several matrices after a layernorm can give every workgroup one matrix only: the workgroup then loads and
-// stages one mixed vector (uint8: one set of ry / my, two sums) instead of all of them.  FRHIP_SEG_EXCLUSIVE=0: off.
-// Measured (decode tok/s, exclusive against shared): RWKV-5.2 3B uint8 845 against 772, RWKV-4 1.5B uint8 1635 against 1594,
-// RWKV-5.2 3B binary16 (four matrices) 741 against 736; binary16 launches of two matrices lose half a percent (1419
-// against 1426: their workgroups stage two 4 KB vectors either way), so those stay shared.  FRHIP_SEG_EXCLUSIVE=0 / 1
-// forces it off / on for every such launch.
+// stages one mixed vector (uint8: one set of ry / my, two sums) instead of all of them, at the price of a longer search
+// for its place in the launch.  It pays from about 14 KB of operands saved per workgroup -- (nseg - 1) x (uint8: mix, ry,
+// my; binary16: mix) x 2 K bytes.  Decode tok/s against the shared form on one box: RWKV-5.2 3B uint8 (K = 2560, four
+// and two matrices: 46 and 15 KB) 809 -> 876; its four-matrix binary16 launch (15 KB) 747 -> 760; RWKV-4 1.5B uint8
+// (K = 2048, two matrices: 12 KB) 1 666 -> 1 656 and binary16 (4 KB) 1 426 -> 1 419, which therefore stay shared.
+// FRHIP_SEG_EXCLUSIVE=0 / 1 forces it off / on for every such launch.
 static bool want_exclusive(const RowsArgs& a, bool u8) {
   static const int forced = getenv("FRHIP_SEG_EXCLUSIVE") ? atoi(getenv("FRHIP_SEG_EXCLUSIVE")) : -1;
   if (a.nseg < 2 || a.prologue != P_LN_MIX || forced == 0) return false;
-  return forced > 0 || u8 || a.nseg >= 3;
+  return forced > 0 || (long)(a.nseg - 1) * (u8 ? 3 : 1) * 2 * a.K >= 14 * 1024;
 }
 
 static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
@@ -1505,34 +1532,39 @@ static int pick_r(const RowsArgs& a, int grid, int nch, bool u8, bool* multi) {
 
 // false when the (R, NCH, MULTI) tiling is not compiled (pick_r never asks for one that is not)
 template <int R, int NCH, bool U8, bool MULTI>
-static void launch_rows_pro(int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
+static void launch_rows_pro(int grid, size_t lds, hipStream_t st, const RowsArgs& a, const ExclArgs* xa) {
   switch (a.prologue) {
     case P_COPY: hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_COPY>), dim3(grid), dim3(kThreads), lds, st, a); break;
     case P_LN: hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_LN>), dim3(grid), dim3(kThreads), lds, st, a); break;
-    default: hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_LN_MIX>), dim3(grid), dim3(kThreads), lds, st, a); break;
+    default:
+      if (xa)
+        hipLaunchKernelGGL((rows_excl_kernel<R, NCH, U8, MULTI>), dim3(grid), dim3(kThreads), lds, st, a, *xa);
+      else
+        hipLaunchKernelGGL((rows_kernel<R, NCH, U8, MULTI, P_LN_MIX>), dim3(grid), dim3(kThreads), lds, st, a);
+      break;
   }
 }
 
 template <int R, int NCH>
-static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
+static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a, const ExclArgs* xa) {
   if (!multi) {
     if constexpr ((R * NCH <= kMaxLoads && R <= 6) || R == 1) {
       if (u8)
-        launch_rows_pro<R, NCH, true, false>(grid, lds, st, a);
+        launch_rows_pro<R, NCH, true, false>(grid, lds, st, a, xa);
       else
-        launch_rows_pro<R, NCH, false, false>(grid, lds, st, a);
+        launch_rows_pro<R, NCH, false, false>(grid, lds, st, a, xa);
       return true;
     }
   } else {
     if constexpr ((R * NCH <= kMaxLoads / 2 && R <= 4) || R == 1) {
       if (u8)
-        launch_rows_pro<R, NCH, true, true>(grid, lds, st, a);
+        launch_rows_pro<R, NCH, true, true>(grid, lds, st, a, xa);
       else
-        launch_rows_pro<R, NCH, false, true>(grid, lds, st, a);
+        launch_rows_pro<R, NCH, false, true>(grid, lds, st, a, xa);
       return true;
     } else if constexpr (R == 8 && NCH <= 2) {
       if (!u8) return false;
-      launch_rows_pro<R, NCH, true, true>(grid, lds, st, a);
+      launch_rows_pro<R, NCH, true, true>(grid, lds, st, a, xa);
       return true;
     }
   }
@@ -1540,15 +1572,16 @@ static bool launch_rows_rn(bool u8, bool multi, int grid, size_t lds, hipStream_
 }
 
 template <int NCH>
-static bool launch_rows_n(int R, bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a) {
+static bool launch_rows_n(int R, bool u8, bool multi, int grid, size_t lds, hipStream_t st, const RowsArgs& a,
+                          const ExclArgs* xa) {
   switch (R) {
-    case 1: return launch_rows_rn<1, NCH>(u8, multi, grid, lds, st, a);
-    case 2: return launch_rows_rn<2, NCH>(u8, multi, grid, lds, st, a);
-    case 3: return launch_rows_rn<3, NCH>(u8, multi, grid, lds, st, a);
-    case 4: return launch_rows_rn<4, NCH>(u8, multi, grid, lds, st, a);
-    case 5: return launch_rows_rn<5, NCH>(u8, multi, grid, lds, st, a);
-    case 6: return launch_rows_rn<6, NCH>(u8, multi, grid, lds, st, a);
-    case 8: return launch_rows_rn<8, NCH>(u8, multi, grid, lds, st, a);
+    case 1: return launch_rows_rn<1, NCH>(u8, multi, grid, lds, st, a, xa);
+    case 2: return launch_rows_rn<2, NCH>(u8, multi, grid, lds, st, a, xa);
+    case 3: return launch_rows_rn<3, NCH>(u8, multi, grid, lds, st, a, xa);
+    case 4: return launch_rows_rn<4, NCH>(u8, multi, grid, lds, st, a, xa);
+    case 5: return launch_rows_rn<5, NCH>(u8, multi, grid, lds, st, a, xa);
+    case 6: return launch_rows_rn<6, NCH>(u8, multi, grid, lds, st, a, xa);
+    case 8: return launch_rows_rn<8, NCH>(u8, multi, grid, lds, st, a, xa);
     default: return false;
   }
 }
@@ -1656,15 +1689,16 @@ static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char
   for (int s = 0; s < kMaxSeg; s++)
     a.bstart[s + 1] = s < a.nseg ? a.bstart[s] + (a.seg[s].w.N + R - 1) / R : INT_MAX;
   a.split = make_split(a.bstart[a.nseg], grid);
-  a.exclusive = 0;
+  ExclArgs xargs;
+  const ExclArgs* xa = nullptr;
   int wgs[kMaxSeg];
   if (want_exclusive(a, u8) && share_workgroups(a, R, grid, wgs)) {
-    a.exclusive = 1;
-    a.wg_start[0] = 0;
+    memset(&xargs, 0, sizeof(xargs));
     for (int s = 0; s < kMaxSeg; s++) {
-      a.wg_start[s + 1] = s < a.nseg ? a.wg_start[s] + wgs[s] : INT_MAX;
-      if (s < a.nseg) a.seg_split[s] = make_split(a.bstart[s + 1] - a.bstart[s], wgs[s]);
+      xargs.wg_start[s + 1] = s < a.nseg ? xargs.wg_start[s] + wgs[s] : INT_MAX;
+      if (s < a.nseg) xargs.seg_split[s] = make_split(a.bstart[s + 1] - a.bstart[s], wgs[s]);
     }
+    xa = &xargs;
   }
   const size_t lds = staged_bytes(nch, u8) * (u8 ? a.nseg : a.nvec);
   FR_TRY(check_lds(lds));
@@ -1673,15 +1707,15 @@ static int launch_rows(const RowsArgs& args, bool u8, hipStream_t st, const char
 #endif
   bool ok = false;
   switch (nch) {
-    case 1: ok = launch_rows_n<1>(R, u8, multi, grid, lds, st, a); break;
-    case 2: ok = launch_rows_n<2>(R, u8, multi, grid, lds, st, a); break;
-    case 3: ok = launch_rows_n<3>(R, u8, multi, grid, lds, st, a); break;
-    case 4: ok = launch_rows_n<4>(R, u8, multi, grid, lds, st, a); break;
-    case 5: ok = launch_rows_n<5>(R, u8, multi, grid, lds, st, a); break;
-    case 8: ok = launch_rows_n<8>(R, u8, multi, grid, lds, st, a); break;
-    case 9: ok = launch_rows_n<9>(R, u8, multi, grid, lds, st, a); break;
-    case 16: ok = launch_rows_n<16>(R, u8, multi, grid, lds, st, a); break;
-    case 18: ok = launch_rows_n<18>(R, u8, multi, grid, lds, st, a); break;
+    case 1: ok = launch_rows_n<1>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 2: ok = launch_rows_n<2>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 3: ok = launch_rows_n<3>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 4: ok = launch_rows_n<4>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 5: ok = launch_rows_n<5>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 8: ok = launch_rows_n<8>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 9: ok = launch_rows_n<9>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 16: ok = launch_rows_n<16>(R, u8, multi, grid, lds, st, a, xa); break;
+    case 18: ok = launch_rows_n<18>(R, u8, multi, grid, lds, st, a, xa); break;
     default: break;
   }
   if (!ok) return set_error(FRHIP_ESHAPE, "row-streaming kernel: no compiled tiling for this shape");
