@@ -163,6 +163,48 @@ def test_kept_binary16_image_of_uint8_weights_gives_the_same_bits(spec, generic)
         assert np.array_equal(a, b)
 
 
+_FORMS_CHILD = r"""
+import hashlib, importlib, os, sys
+import numpy as np
+sys.path.insert(0, sys.argv[1])
+fr = importlib.import_module("faster-rwkv_amd")
+for spec, strategy in [("v=5.2,L=2,C=2560,F=8960,V=4096,H=40,seed=31", "hip int8"),
+                       ("v=5.2,L=2,C=2560,F=8960,V=4096,H=40,seed=31", "hip fp16"),
+                       ("v=4,L=2,C=2048,F=8192,V=4096,seed=32", "hip int8"),
+                       ("v=5,L=2,C=768,F=2688,V=4096,H=12,seed=33", "hip fp16")]:
+    m = fr.Model("synthetic:" + spec, strategy)
+    h = hashlib.sha1()
+    tok = 7
+    for _ in range(6):
+        lg = m.run(tok)
+        h.update(lg.tobytes())
+        tok = int(np.argmax(lg))
+    m.close()
+    print(h.hexdigest())
+"""
+
+
+def test_one_matrix_per_workgroup_and_shared_launches_give_the_same_bits():
+    """The layernorm launches of several matrices exist in two forms (every workgroup serving all matrices, or one:
+    rows_excl_kernel); which one runs is a matter of speed only.  FRHIP_SEG_EXCLUSIVE=0 / 1 forces the form for
+    every such launch (read once per process, hence the child processes): same logits, bit for bit, as the default
+    choice, for RWKV-5.2 at the 3B width (where the default picks the one-matrix form), RWKV-4 at the 1.5B width
+    and a narrow RWKV-5.0 (where it does not)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    seen = {}
+    for form in (None, "0", "1"):
+        env = {k: v for k, v in os.environ.items() if k != "FRHIP_SEG_EXCLUSIVE"}
+        if form is not None:
+            env["FRHIP_SEG_EXCLUSIVE"] = form
+        out = subprocess.run([sys.executable, "-c", _FORMS_CHILD, root], env=env, capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        seen[form] = out.stdout.split()
+        assert len(seen[form]) == 4
+    assert seen[None] == seen["0"] == seen["1"]
+
+
 @pytest.mark.parametrize("spec,strategy", [
     ("v=4,L=4,C=512,F=2048,V=4096,seed=21", "hip fp16"),
     ("v=4,L=4,C=512,F=2048,V=4096,seed=21", "hip int8"),
